@@ -1,0 +1,163 @@
+#!/usr/bin/env python3
+"""Benchmark of the W8A8 matmul-reduce-scatter shard on one MI355X.
+
+A step is one launch of the fused kernel over one batch of synthetic input:
+BASELINE config 4, A[8192,1792] int8, B[1792,4096] int8, per-token / per-channel fp32 scales,
+7 staged fp32 peer partials of the kept block, kept output [1024,4096] bf16.  Inputs are resident
+in HBM before the timed region.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode kept|outbound] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
+
+
+def cpu_baseline(M, N, K, P, rank, repeats):
+    """The CPU oracle (a port of the reference's golden math) on the same workload, all host threads."""
+    import numpy as np
+    import oracle
+    rng = np.random.default_rng(20250101)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    run = lambda: oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, rank * rows, rows, peers, oracle.BF16,
+                                                     want_acc=False)
+    run()  # warm-up
+    ts = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        run()
+        ts.append(time.perf_counter() - t0)
+    best = min(ts)
+    return {"value": 2.0 * M * N * K / best / 1e12, "unit": "TOPS", "cores": oracle.num_threads(), "kind": "port",
+            "sample": "full workload (M=%d,K=%d,N=%d,P=%d), 1 warm-up + %d timed runs, best %.3f s, mean %.3f s; "
+                      "OpenMP over rows, gcc -O3 -march=native -ffp-contract=off" % (M, K, N, P, repeats, best,
+                                                                                    sum(ts) / len(ts))}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--mode", choices=["kept", "outbound"], default="kept",
+                    help="kept: non-kept tiles are folded into checksums (BASELINE's literal outputs); "
+                         "outbound: they are also stored as fp32 to the symmetric workspace")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-repeats", type=int, default=5)
+    ap.add_argument("--rank", type=int, default=0)
+    ap.add_argument("--m0", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU (peers are staged in the same GPU's HBM); --gpus %d is not "
+              "supported, use --gpus 1" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import ctypes as C
+    import torch
+    from mm_rs_with_catlass_amd import lib as L
+    from mm_rs_with_catlass_amd import ops
+    L.load()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = "cuda:0"
+    M, K, N, P, rank = 8192, 1792, 4096, 8, args.rank
+    rows = M // P
+    g = torch.Generator(device=dev).manual_seed(20250101)
+    x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
+    x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
+    s1 = torch.empty(M, device=dev).uniform_(0.005, 0.02, generator=g)
+    s2 = torch.empty(N, device=dev).uniform_(0.001, 0.01, generator=g)
+    peers = [torch.randn((rows, N), device=dev, generator=g) for _ in range(P - 1)]
+    out = torch.empty((rows, N), dtype=torch.bfloat16, device=dev)
+    tiling = ops.default_tiling(M, K, N, P, m0=args.m0, n0=0, k0=0)
+    desc0 = L.make_desc(rank, P, [16] * (P - 1))
+    ntasks = L.load().catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(tiling), C.byref(desc0))
+    kw = {}
+    if args.mode == "outbound":
+        need = L.load().catcoc_get_workspace_size(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, C.byref(tiling), C.byref(desc0))
+        kw["outbound"] = torch.empty(need // 4, dtype=torch.float32, device=dev)
+    else:
+        kw["checksum"] = torch.zeros(ntasks, dtype=torch.int64, device=dev)
+
+    # arguments are validated and bound once; a step is one call of the C-ABI launcher
+    step, _ = ops.prepare_quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, rank, P, tiling=tiling, out=out, **kw)
+    step()
+    L.check()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # per-launch HIP events on the launch stream (torch's current stream), inside the timed region
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for a, b in evs:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kern_ms = [a.elapsed_time(b) for a, b in evs]
+    avg_kernel_s = sum(kern_ms) / len(kern_ms) / 1e3
+    ms_per_step = wall / args.steps * 1e3
+
+    # bounded parity check of the timed configuration: a row sample of the kept block against the oracle
+    import numpy as np
+    import oracle
+    sel = np.arange(0, rows, 97)
+    _, want = oracle.quant_matmul_reduce_scatter(
+        x1[rank * rows + sel].cpu().numpy(), x2.cpu().numpy(), s1[rank * rows + sel].cpu().numpy(), s2.cpu().numpy(),
+        None, 0, len(sel), [p[sel].cpu().numpy() for p in peers], oracle.BF16, want_acc=False)
+    got = out[sel].view(torch.int16).cpu().numpy().view(np.uint16)
+    parity_ok = bool(np.array_equal(got, want))
+
+    ops_per_step = 2.0 * M * N * K
+    alg_bytes = M * K + K * N + 4 * (M + N) + (P - 1) * rows * N * 4 + rows * N * 2
+    if args.mode == "outbound":
+        alg_bytes += (P - 1) * rows * N * 4
+    value = ops_per_step / (wall / args.steps) / 1e12
+    achieved = ops_per_step / avg_kernel_s / 1e12
+    info = ops.device_info()
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("quant_rs_config4_" + args.mode)
+        except Exception:
+            traffic = None
+    line = {
+        "metric": "W8A8 matmul-RS shard int8 TOPS + % MFMA/HBM roofline, 1 MI355X",
+        "value": round(value, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "W8A8 quant matmul-reduce-scatter shard (BASELINE config 4): M=8192 K=1792 N=4096 "
+                               "P=8 rank=%d, int8 x int8 -> int32, dequant, +7 staged fp32 peers, bf16 [1024,4096]" % rank,
+                   "mode": args.mode, "tile": "%dx256x64" % (tiling.m0 or 128), "tasks": int(ntasks),
+                   "parity_sample_ok": parity_ok},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                     "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": traffic,
+                     "kernel_us_avg": round(avg_kernel_s * 1e6, 2), "kernel_us_min": round(min(kern_ms) * 1e3, 2),
+                     "algorithmic_bytes": int(alg_bytes),
+                     "hbm_frac_at_algorithmic_bytes": round(alg_bytes / avg_kernel_s / 1e9 / PEAK_HBM_GBS, 4)},
+        "device": info,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(M, N, K, P, rank, args.cpu_repeats)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

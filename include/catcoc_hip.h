@@ -1,0 +1,264 @@
+/*
+ * catcoc_hip.h -- C ABI of libcatcoc_hip.so: the per-rank fused GEMM path of
+ * CATCOC (tile GEMM + dequant + peer-partial reduce epilogue) for AMD MI355X
+ * (gfx950), on ONE GPU.  Peer ranks' data are buffers staged in this GPU's HBM.
+ *
+ * Every entry point names the reference interface it stands in for (paths are
+ * relative to the reference tree).  Plain C types only; `stream` is a
+ * hipStream_t passed as void*.  All launches are asynchronous on `stream`; the
+ * caller owns every buffer and the library allocates nothing on a launch.
+ */
+#ifndef CATCOC_HIP_H
+#define CATCOC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CATCOC_API __attribute__((visibility("default")))
+
+/* ----------------------------------------------------------------------- */
+/* Types kept binary-identical to the reference                              */
+/* ----------------------------------------------------------------------- */
+
+/* examples/dynamic_tiling/include/info.h:29-42 -- twelve uint32_t, same order.
+ * m,k,n: problem (for ALLGATHER_MATMUL m is the rows of ONE rank's shard).
+ * m0,n0,k0: workgroup macro tile; 0 lets the library choose.
+ * commInterval x blockNum: tiles per scheduling round (blockNum, the
+ * reference's BLOCK_NUM = 20 AI cores, comes from CatcocSymmetricDesc).
+ * commTileM, commBlockM, commNpuSplit, commDataSplit: comm-epilogue chunking of
+ * the reference; accepted, validated like the reference does, and otherwise
+ * unused because the reduce runs in registers in the GEMM's own epilogue. */
+typedef struct CocTilingParams {
+    uint32_t m;
+    uint32_t k;
+    uint32_t n;
+    uint32_t m0;
+    uint32_t k0;
+    uint32_t n0;
+    uint32_t commTileM;
+    uint32_t commInterval;
+    uint32_t commNpuSplit;
+    uint32_t commDataSplit;
+    uint32_t commBlockM;
+    uint32_t rankSize;
+} CocTilingParams;
+
+/* examples/dynamic_tiling/include/launch_map.h:6-11 (values 0..2 unchanged). */
+typedef enum CocCommType {
+    MATMUL_ALLREDUCE = 0,
+    ALLGATHER_MATMUL = 1,
+    MATMUL_REDUCE_SCATTER = 2,
+    QUANT_MATMUL_REDUCE_SCATTER = 3, /* examples/02_matmul_reduce_scatter/quant_matmul_reduce_scatter.cpp */
+    TYPE_NUM
+} CocCommType;
+
+/* examples/dynamic_tiling/include/launch_map.h:13-16; INT8 = 2 is the ACL code. */
+typedef enum CocDataType {
+    FP16 = 1,
+    INT8 = 2,
+    BF16 = 27
+} CocDataType;
+
+/* examples/dynamic_tiling/include/launch_map.h:18-19  KernelFuncPtr.  The C++
+ * reference passes `CocTilingParams &`; at the ABI level that is this pointer.
+ * aW, bW are reserved and ignored (examples/dynamic_tiling/impl/kernel_fp16.cpp:29-30).
+ * fftsAddr is accepted and ignored (no cross-core flags on a GPU).
+ *   MATMUL_ALLREDUCE     : a [m,k], b [k,n], c [m,n]
+ *   ALLGATHER_MATMUL     : a [m,k] = this rank's shard, b [k,n], c [m*rankSize,n]
+ *   MATMUL_REDUCE_SCATTER: a [m,k], b [k,n], c [m/rankSize,n]
+ * transA / transB != 0 mean the operand is stored transposed ([k,m] / [n,k]),
+ * the ColumnMajor instantiations of kernel_fp16.cpp:31-43.
+ * symmetricPtr points at a CatcocSymmetricDesc in HOST memory (see below). */
+typedef void (*CatcocKernelFuncPtr)(void *stream, uint64_t fftsAddr, uint8_t *a, uint8_t *b, uint8_t *c,
+                                    uint8_t *aW, uint8_t *bW, uint8_t *symmetricPtr, CocTilingParams *tiling,
+                                    uint32_t transA, uint32_t transB);
+
+/* ----------------------------------------------------------------------- */
+/* One-GPU stand-in for the symmetric heap                                   */
+/* ----------------------------------------------------------------------- */
+
+#define CATCOC_MAX_RANKS 16
+#define CATCOC_DESC_MAGIC 0x43544343u /* "CCTC" */
+
+/* What happens to tiles whose rows belong to another rank (the reference stores
+ * them to the symmetric workspace, quant_matmul_reduce_scatter.hpp:196-201). */
+#define CATCOC_OUTBOUND_CHECKSUM 0u /* fold each tile's accumulators into `checksum` (keeps the MACs observable) */
+#define CATCOC_OUTBOUND_STORE 1u    /* store the tile to `outbound` in the reference's tile-linear layout, as fp32
+                                       (dequantised for W8A8), or int32 when CATCOC_FLAG_REDUCE_INT32 is set */
+#define CATCOC_OUTBOUND_MASK 0x3u
+/* W8A8 only: peers hold int32 partials that are added BEFORE the dequant (the
+ * reference's order, quant_matmul_reduce_scatter.hpp:285-351); default is fp32
+ * partials added after the dequant. */
+#define CATCOC_FLAG_REDUCE_INT32 0x4u
+/* Keep the linear workgroup -> task order (no XCD-aware chunking). */
+#define CATCOC_FLAG_LINEAR_ORDER 0x8u
+
+/* Replaces the reference's `symmetricPtr` workspace + shmem_my_pe()/shmem_n_pes()
+ * (examples/dynamic_tiling/impl/kernel/matmul_reduce_scatter.h:155-156): which
+ * rank this GPU plays and where the other ranks' staged data live.  Zero-filled
+ * fields take the documented defaults. */
+typedef struct CatcocSymmetricDesc {
+    uint32_t magic;           /* CATCOC_DESC_MAGIC */
+    uint32_t rankIdx;         /* shmem_my_pe() */
+    uint32_t rankSize;        /* shmem_n_pes(); must match tiling.rankSize when that is non-zero */
+    uint32_t blockNum;        /* BLOCK_NUM of the schedule; 0 = 256 (one per CU) */
+    uint32_t workspaceStages; /* WORKSPACE_STAGES; 0 = 2 */
+    uint32_t swizzleOffset;   /* GemmIdentityBlockSwizzle<offset,direction>; 0 = <7,1> as in every example */
+    uint32_t swizzleDirection;
+    uint32_t flags;           /* CATCOC_OUTBOUND_* | CATCOC_FLAG_* */
+    uint32_t keptRowBegin;    /* explicit kept row range of the reduce-scatter; both 0 = rows */
+    uint32_t keptRows;        /*   [rankIdx*m/rankSize, +m/rankSize) as in the reference */
+    uint32_t splitK;          /* skinny-M path: k slices; 0 = GetSplitkFactor heuristic */
+    uint32_t reserved0;
+    /* Reduce paths: peers[s], s = 0..rankSize-2, are the other ranks' partial
+     * results for this rank's kept rows (fp32, or int32 with REDUCE_INT32), added
+     * in slot order after the local partial.  Row `peerRowOffset + i` of a peer
+     * buffer lines up with kept row i; peerLd is its leading dimension in elements.
+     * ALLGATHER_MATMUL: peers[s] are the other ranks' A shards in ascending rank
+     * order (this rank's own shard is the `a` argument), each [m,k], read in place. */
+    const void *peers[CATCOC_MAX_RANKS];
+    int64_t peerLd;
+    int64_t peerRowOffset;
+    void *outbound;           /* OUTBOUND_STORE target, rows (stage*blockPerComm + blockIdxInComm)*m0, n0 columns */
+    uint64_t outboundBytes;   /* capacity of `outbound` */
+    int64_t *checksum;        /* OUTBOUND_CHECKSUM target: one int64 per task (W8A8) / one double per task (float) */
+    void *accDump;            /* optional full [m,n] int32 (W8A8) or fp32 (float) local partial, for bit-exact checks */
+    void *splitkWorkspace;    /* skinny-M path: int32 [m,n] + one uint32 per tile, zeroed by the caller once */
+    uint64_t splitkWorkspaceBytes;
+} CatcocSymmetricDesc;
+
+/* ----------------------------------------------------------------------- */
+/* Registry and launchers                                                    */
+/* ----------------------------------------------------------------------- */
+
+/* KernelDispatcher::GetKernelFunc (examples/dynamic_tiling/include/launch_map.h:35-42).
+ * Returns NULL for an unregistered (commType, dataType) pair, as the reference does. */
+CATCOC_API CatcocKernelFuncPtr catcoc_get_kernel(int commType, int dataType);
+
+/* LaunchMatmulAllReduceFP16 / BF16      (examples/dynamic_tiling/impl/kernel_fp16.cpp:22-44, kernel_bf16.cpp) */
+CATCOC_API void catcoc_launch_matmul_allreduce_fp16(void *stream, uint64_t fftsAddr, uint8_t *a, uint8_t *b,
+    uint8_t *c, uint8_t *aW, uint8_t *bW, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA,
+    uint32_t transB);
+CATCOC_API void catcoc_launch_matmul_allreduce_bf16(void *stream, uint64_t fftsAddr, uint8_t *a, uint8_t *b,
+    uint8_t *c, uint8_t *aW, uint8_t *bW, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA,
+    uint32_t transB);
+/* LaunchAllGatherMatmulFP16 / BF16      (kernel_fp16.cpp:46-62) */
+CATCOC_API void catcoc_launch_allgather_matmul_fp16(void *stream, uint64_t fftsAddr, uint8_t *a, uint8_t *b,
+    uint8_t *c, uint8_t *aW, uint8_t *bW, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA,
+    uint32_t transB);
+CATCOC_API void catcoc_launch_allgather_matmul_bf16(void *stream, uint64_t fftsAddr, uint8_t *a, uint8_t *b,
+    uint8_t *c, uint8_t *aW, uint8_t *bW, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA,
+    uint32_t transB);
+/* LaunchMatmulReduceScatterFP16 / BF16  (kernel_fp16.cpp:64-86) */
+CATCOC_API void catcoc_launch_matmul_reduce_scatter_fp16(void *stream, uint64_t fftsAddr, uint8_t *a, uint8_t *b,
+    uint8_t *c, uint8_t *aW, uint8_t *bW, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA,
+    uint32_t transB);
+CATCOC_API void catcoc_launch_matmul_reduce_scatter_bf16(void *stream, uint64_t fftsAddr, uint8_t *a, uint8_t *b,
+    uint8_t *c, uint8_t *aW, uint8_t *bW, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA,
+    uint32_t transB);
+
+/* ShmemQuantMatmulReduceScatter<<<...>>>(fftsAddr, x1, x2, scale_x1, scale_x2, bias, c_accum, d_out,
+ * symmetricPtr, m, n, k)   (examples/02_matmul_reduce_scatter/quant_matmul_reduce_scatter.cpp:54-60).
+ * x1 [m,k] int8, x2 [k,n] int8, scale_x1 [m] fp32 per token, scale_x2 [n] fp32 per channel,
+ * bias [n] int32 or NULL, c_accum [m/P,n] int32 or NULL (receives the kept block's local
+ * accumulators incl. bias), d_out [m/P,n].  Fixed configuration of the example:
+ * tile 128x256, commInterval 10, swizzle <7,1>; rank and rankSize come from the descriptor.
+ * d_out is bf16 (the kernel's ElementD, quant_matmul_reduce_scatter.hpp:48). */
+CATCOC_API void catcoc_quant_matmul_reduce_scatter(void *stream, uint64_t fftsAddr, uint8_t *x1, uint8_t *x2,
+    uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum, uint8_t *d_out, uint8_t *symmetricPtr,
+    uint32_t m, uint32_t n, uint32_t k);
+
+/* Same operator driven by CocTilingParams, as the dynamic_tiling wrappers do for the float ops
+ * (examples/dynamic_tiling/impl/kernel/matmul_reduce_scatter.h:126-170).  outDataType is FP16 or
+ * BF16 (the example instantiates the dequant epilogue with half, quant_matmul_reduce_scatter.cpp:129). */
+CATCOC_API void catcoc_launch_quant_matmul_reduce_scatter(void *stream, uint64_t fftsAddr, uint8_t *x1, uint8_t *x2,
+    uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum, uint8_t *d_out, uint8_t *symmetricPtr,
+    CocTilingParams *tiling, uint32_t transA, uint32_t transB, uint32_t outDataType);
+
+/* ----------------------------------------------------------------------- */
+/* Validation, errors, sizes                                                 */
+/* ----------------------------------------------------------------------- */
+
+/* The launchers return void like the reference's; a rejected call launches nothing and records
+ * an error.  catcoc_last_error(): message of the calling thread's last rejected call ("" if none);
+ * catcoc_last_status(): 0 = the last call on this thread was accepted. */
+CATCOC_API const char *catcoc_last_error(void);
+CATCOC_API int catcoc_last_status(void);
+
+/* Catlass::Status-style pre-flight check (3rdparty/catlass/include/catlass/gemm/device/device_gemm.hpp:46-53):
+ * 0 if the launcher would accept these arguments, else non-zero with catcoc_last_error() set. */
+CATCOC_API int catcoc_can_implement(int commType, int dataType, const CocTilingParams *tiling,
+                                    const CatcocSymmetricDesc *desc, uint32_t transA, uint32_t transB);
+
+/* Bytes of `outbound` needed for OUTBOUND_STORE with this tiling / descriptor (the reference
+ * sizes layoutSymmetric = m0*commInterval*BLOCK_NUM*WORKSPACE_STAGES x n0, matmul_reduce_scatter.h:161). */
+CATCOC_API uint64_t catcoc_get_workspace_size(int commType, int dataType, const CocTilingParams *tiling,
+                                              const CatcocSymmetricDesc *desc);
+
+/* Number of tasks (tiles) a launch runs; `checksum` needs this many entries. */
+CATCOC_API uint32_t catcoc_get_task_count(int commType, const CocTilingParams *tiling,
+                                          const CatcocSymmetricDesc *desc);
+
+/* ----------------------------------------------------------------------- */
+/* dynamic_tiling host logic                                                 */
+/* ----------------------------------------------------------------------- */
+
+/* GetTilings (examples/dynamic_tiling/include/tiling.h:83-105): fills `out` (capacity maxOut) with the
+ * candidates of the 5x5x2 search space that pass the op's check; returns how many exist. */
+CATCOC_API int catcoc_get_tilings(const CocTilingParams *base, int commType, int rankSize, int blockNum,
+                                  CocTilingParams *out, int maxOut);
+/* CheckCommIntervalReduceScatter / AllReduce / AllGather (tiling.h:32-62); 1 = valid. */
+CATCOC_API int catcoc_check_comm_interval_reduce_scatter(const CocTilingParams *t, int rankSize, int blockNum);
+CATCOC_API int catcoc_check_comm_interval_allreduce(const CocTilingParams *t, int rankSize, int blockNum);
+CATCOC_API int catcoc_check_comm_interval_allgather(const CocTilingParams *t, int rankSize);
+/* SplitkMatmul::GetSplitkFactor (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:219-265). */
+CATCOC_API uint32_t catcoc_get_splitk_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t coreNum, uint32_t m0,
+                                             uint32_t n0, uint32_t k0);
+/* The defaults dynamic_tiling.cpp:215-227 fills in before the search (m0,k0,n0 = 128,256,256; commTileM 64;
+ * commInterval 20; npuSplit 1; dataSplit 2; commBlockM 64). */
+CATCOC_API void catcoc_default_tiling(CocTilingParams *t, uint32_t m, uint32_t k, uint32_t n, uint32_t rankSize);
+
+/* ----------------------------------------------------------------------- */
+/* Block schedulers (the same integer code the kernels run, callable on the host) */
+/* ----------------------------------------------------------------------- */
+
+/* GemmIdentityBlockSwizzle<off,dir>::GetBlockCoord on a loopsM x loopsN tile grid
+ * (3rdparty/catlass/include/catlass/gemm/block/block_swizzle.hpp:79-113). */
+CATCOC_API void catcoc_swizzle_block_coord(uint32_t off, uint32_t dir, uint32_t loopsM, uint32_t loopsN,
+                                           uint32_t task, uint32_t *mIdx, uint32_t *nIdx);
+/* SplitkGemmIdentityBlockSwizzle::GetBlockCoord / slice k extent (block_swizzle.hpp:151-235). */
+CATCOC_API void catcoc_splitk_block_coord(uint32_t off, uint32_t dir, uint32_t loopsM, uint32_t loopsN,
+                                          uint32_t kTiles, uint32_t f, uint32_t task, uint32_t *mIdx,
+                                          uint32_t *nIdx, uint32_t *kIdx, uint32_t *slice);
+CATCOC_API uint32_t catcoc_splitk_actual_k(uint32_t K, uint32_t k0, uint32_t f, uint32_t slice);
+/* GemmIdentityBlockSwizzleAllGather::GetBlockCoord (include/catcoc/dgemm/block/block_swizzle_allgather.hpp:88-108). */
+CATCOC_API void catcoc_allgather_block_coord(uint32_t off, uint32_t dir, uint32_t P, uint32_t commInterval,
+                                             uint32_t loopsMRank, uint32_t loopsN, uint32_t task, uint32_t *mIdx,
+                                             uint32_t *nIdx);
+/* BlockCommSwizzle<dir>::GetBlockIdx (include/catcoc/comm_epilogue/block/comm_block_swizzle.hpp:147-186). */
+CATCOC_API void catcoc_comm_block_idx(uint32_t dir, uint32_t P, uint32_t splitRow, uint32_t splitCol,
+                                      uint32_t dataLoopsInRank, uint32_t task, uint32_t *dataIdx,
+                                      uint32_t *rankIdx);
+/* The tile a task computes in each operator (quant_matmul_reduce_scatter.hpp:172-201,
+ * matmul_allreduce.hpp:154-179, allgather_matmul.hpp:142-163): target rank, first row/col of the tile in
+ * the global problem, and the workspace row of the reference's tile-linear layout.  Returns 0 past the end. */
+CATCOC_API int catcoc_task_tile(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
+                                uint32_t task, uint32_t *targetRank, uint32_t *row, uint32_t *col,
+                                uint32_t *wsRow);
+/* The task workgroup `wg` of a launch with `tasks` tasks runs (XCD-aware chunking unless
+ * CATCOC_FLAG_LINEAR_ORDER); a bijection on [0,tasks). */
+CATCOC_API uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags);
+
+/* Library / device information: fills cuCount, clockMHz of the current device; returns 0 on success. */
+CATCOC_API int catcoc_device_info(int *cuCount, int *clockMHz, char *name, int nameLen);
+CATCOC_API const char *catcoc_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CATCOC_HIP_H */

@@ -1,0 +1,480 @@
+// C ABI of libcatcoc_hip.so: argument validation, tiling selection and dispatch
+// to the fused GEMM kernels.  Declarations and the reference interfaces they
+// replace are in include/catcoc_hip.h.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "catcoc_hip.h"
+#include "gemm_args.h"
+#include "tile_sched.h"
+
+namespace catcoc {
+int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream);
+int launch_gemm_f16(const GemmArgs &args, int variant, bool edge, void *stream);
+int launch_gemm_bf16(const GemmArgs &args, int variant, bool edge, void *stream);
+
+static int launch_gemm(uint32_t dtype, const GemmArgs &args, int variant, bool edge, void *stream)
+{
+    switch (dtype) {
+        case DT_I8: return launch_gemm_i8(args, variant, edge, stream);
+        case DT_F16: return launch_gemm_f16(args, variant, edge, stream);
+        case DT_BF16: return launch_gemm_bf16(args, variant, edge, stream);
+        default: return (int)hipErrorInvalidValue;
+    }
+}
+}
+
+using namespace catcoc;
+
+namespace {
+
+thread_local char g_err[512] = "";
+thread_local int g_status = 0;
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    g_status = code;
+    return code;
+}
+
+void ok()
+{
+    g_err[0] = 0;
+    g_status = 0;
+}
+
+enum { E_NULL = 1, E_DESC = 2, E_SHAPE = 3, E_RANK = 4, E_TILING = 5, E_DTYPE = 6, E_WORKSPACE = 7, E_LAUNCH = 8 };
+
+constexpr uint32_t kDefaultBlockNum = 256;  // one scheduling slot per CU of an MI355X
+constexpr uint32_t kDefaultStages = 2;      // WORKSPACE_STAGES, examples/dynamic_tiling/include/info.h:18
+
+struct Plan {
+    GemmArgs args;
+    int variant;  // 0 = general kernel, else tile rows / 64 of the fast kernel
+    bool edge;
+    uint32_t dtype;
+    uint32_t blockNum;
+};
+
+uint32_t elem_size(uint32_t dt) { return dt == DT_I8 ? 1u : 2u; }
+
+// Everything a launcher checks before it launches; fills `plan` except the buffer pointers.
+int make_plan(int commType, int dataType, const CocTilingParams *t, const CatcocSymmetricDesc *d, uint32_t transA,
+              uint32_t transB, Plan &plan)
+{
+    if (t == nullptr) return fail(E_NULL, "tiling is NULL");
+    if (d == nullptr) return fail(E_NULL, "symmetricPtr is NULL (it must point at a CatcocSymmetricDesc)");
+    if (d->magic != CATCOC_DESC_MAGIC) return fail(E_DESC, "symmetricPtr does not point at a CatcocSymmetricDesc (bad magic)");
+    if (commType < 0 || commType >= TYPE_NUM) return fail(E_DTYPE, "unknown commType %d", commType);
+    const bool quant = commType == QUANT_MATMUL_REDUCE_SCATTER;
+    if (quant ? dataType != INT8 : (dataType != FP16 && dataType != BF16))
+        return fail(E_DTYPE, "dataType %d is not registered for commType %d", dataType, commType);
+    if (t->m == 0 || t->n == 0 || t->k == 0) return fail(E_SHAPE, "empty problem m=%u n=%u k=%u", t->m, t->n, t->k);
+    const uint32_t P = d->rankSize;
+    if (P == 0 || P > CATCOC_MAX_RANKS) return fail(E_RANK, "rankSize %u out of range 1..%d", P, CATCOC_MAX_RANKS);
+    if (t->rankSize != 0 && t->rankSize != P) return fail(E_RANK, "tiling.rankSize %u != descriptor rankSize %u", t->rankSize, P);
+    if (d->rankIdx >= P) return fail(E_RANK, "rankIdx %u >= rankSize %u", d->rankIdx, P);
+
+    const uint32_t op = (commType == MATMUL_ALLREDUCE) ? OP_ALLREDUCE : (commType == ALLGATHER_MATMUL) ? OP_ALLGATHER : OP_REDUCE_SCATTER;
+    if (op == OP_REDUCE_SCATTER && t->m % P != 0)
+        return fail(E_SHAPE, "reduce-scatter needs m %% rankSize == 0 (m=%u, rankSize=%u)", t->m, P);
+
+    const uint32_t blockNum = d->blockNum ? d->blockNum : kDefaultBlockNum;
+    const uint32_t stages = d->workspaceStages ? d->workspaceStages : kDefaultStages;
+    const uint32_t commInterval = t->commInterval ? t->commInterval : 1u;
+    // examples/dynamic_tiling/include/tiling.h:32-41: a round's tiles are dealt evenly to the ranks
+    if (op == OP_REDUCE_SCATTER && ((uint64_t)blockNum * commInterval) % P != 0)
+        return fail(E_TILING, "blockNum*commInterval = %u*%u is not a multiple of rankSize %u", blockNum, commInterval, P);
+    const uint32_t off = d->swizzleOffset ? d->swizzleOffset : 7u;
+    const uint32_t dir = d->swizzleOffset ? d->swizzleDirection : 1u;
+    if (dir > 1) return fail(E_TILING, "swizzleDirection %u must be 0 or 1", dir);
+
+    const uint32_t dt = (uint32_t)dataType;
+    const uint32_t es = elem_size(dt);
+    const uint32_t che = 16 / es;
+    const uint32_t mRank = op == OP_REDUCE_SCATTER ? t->m / P : t->m;
+
+    // tile selection: the fast kernel has n0 = 256 and m0 in {64,128}
+    uint32_t m0 = t->m0, n0 = t->n0;
+    if (n0 == 0) n0 = 256;
+    if (m0 == 0) m0 = (mRank <= 64) ? 64 : 128;
+    const bool fastShape = n0 == 256 && (m0 == 64 || m0 == 128) && !transA && t->k % che == 0 && t->n % 4 == 0;
+    plan.variant = fastShape ? (int)(m0 / 64) : 0;
+    plan.edge = !(mRank % m0 == 0 && t->n % n0 == 0 && t->k % (64 / es) == 0);
+    plan.dtype = dt;
+    plan.blockNum = blockNum;
+
+    GemmArgs &a = plan.args;
+    memset(&a, 0, sizeof(a));
+    a.M = t->m;
+    a.N = t->n;
+    a.K = t->k;
+    a.lda = transA ? t->m : t->k;
+    a.ldb = transB ? t->k : t->n;
+    a.ldd = t->n;
+    a.transA = transA ? 1 : 0;
+    a.transB = transB ? 1 : 0;
+    a.outDtype = dt == DT_I8 ? DT_BF16 : dt;
+    a.sched = make_sched(op, t->m, t->n, P, m0, n0, blockNum, commInterval, stages, off, dir);
+    if (a.sched.coreLoops == 0) return fail(E_SHAPE, "no tiles to compute");
+
+    if ((d->flags & CATCOC_OUTBOUND_MASK) == CATCOC_OUTBOUND_STORE) a.flags |= GF_OUTBOUND_STORE;
+    if (d->flags & CATCOC_FLAG_REDUCE_INT32) {
+        if (!quant) return fail(E_DESC, "CATCOC_FLAG_REDUCE_INT32 only applies to the W8A8 operator");
+        a.flags |= GF_REDUCE_INT32;
+    }
+    if (d->flags & CATCOC_FLAG_LINEAR_ORDER) a.flags |= GF_LINEAR_ORDER;
+
+    // kept rows
+    if (op == OP_REDUCE_SCATTER) {
+        a.keptBegin = d->rankIdx * mRank;
+        a.keptRows = mRank;
+        if (d->keptRows != 0 && (d->keptRowBegin != a.keptBegin || d->keptRows != a.keptRows))
+            return fail(E_DESC, "explicit kept rows [%u,+%u) differ from the rank's block [%u,+%u); use the skinny-M entry for that",
+                        d->keptRowBegin, d->keptRows, a.keptBegin, a.keptRows);
+    } else if (op == OP_ALLREDUCE) {
+        a.keptBegin = 0;
+        a.keptRows = t->m;
+    } else {
+        a.keptBegin = 0;
+        a.keptRows = t->m * P;
+    }
+
+    // peers
+    const uint32_t nPeers = P - 1;
+    if (op == OP_ALLGATHER) {
+        a.nPeers = 0;
+        uint32_t s = 0;
+        for (uint32_t r = 0; r < P; ++r) {
+            if (r == d->rankIdx) continue;
+            if (d->peers[s] == nullptr) return fail(E_NULL, "all-gather needs %u peer shards; peers[%u] is NULL", nPeers, s);
+            a.a[r] = d->peers[s++];
+        }
+    } else {
+        a.nPeers = nPeers;
+        for (uint32_t s = 0; s < nPeers; ++s) {
+            if (d->peers[s] == nullptr) return fail(E_NULL, "reduce needs %u staged peer partials; peers[%u] is NULL", nPeers, s);
+            a.peers[s] = d->peers[s];
+        }
+        a.peerLd = d->peerLd ? d->peerLd : t->n;
+        a.peerRowOffset = d->peerRowOffset;
+        if (nPeers && a.peerLd < (int64_t)t->n) return fail(E_DESC, "peerLd %lld < n %u", (long long)a.peerLd, t->n);
+        if (a.peerRowOffset < 0) return fail(E_DESC, "peerRowOffset must be >= 0");
+        if (fastShape && nPeers && (a.peerLd % 4 != 0)) plan.variant = 0;  // 16-byte peer loads need aligned rows
+    }
+
+    if (a.flags & GF_OUTBOUND_STORE) {
+        if (op == OP_REDUCE_SCATTER && P > 1) {
+            if (d->outbound == nullptr) return fail(E_NULL, "CATCOC_OUTBOUND_STORE needs an outbound buffer");
+            const uint64_t need = (uint64_t)stages * a.sched.blockPerComm * m0 * n0 * 4u;
+            if (d->outboundBytes < need)
+                return fail(E_WORKSPACE, "outbound buffer too small: %llu < %llu bytes", (unsigned long long)d->outboundBytes,
+                            (unsigned long long)need);
+        }
+        a.outbound = d->outbound;
+    } else {
+        a.checksum = d->checksum;
+    }
+    a.accDump = d->accDump;
+    return 0;
+}
+
+int check_ptr_align(const Plan &p, const void *a, const void *b)
+{
+    if (p.variant == 0) return 1;
+    const uint32_t es = elem_size(p.dtype);
+    bool okA = ((uintptr_t)a % 16 == 0) && ((p.args.lda * es) % 16 == 0);
+    bool okB = p.args.transB ? (((uintptr_t)b % 16 == 0) && ((p.args.ldb * es) % 16 == 0))
+                             : (((uintptr_t)b % (4 * es) == 0) && (p.args.ldb % 4 == 0));
+    for (uint32_t r = 0; r < p.args.sched.P && okA; ++r)
+        if (p.args.a[r] && (uintptr_t)p.args.a[r] % 16 != 0) okA = false;
+    return okA && okB;
+}
+
+void launch_float(int commType, int dataType, void *stream, uint8_t *a, uint8_t *b, uint8_t *c, uint8_t *symmetricPtr,
+                  CocTilingParams *tiling, uint32_t transA, uint32_t transB)
+{
+    Plan p;
+    const CatcocSymmetricDesc *d = (const CatcocSymmetricDesc *)symmetricPtr;
+    if (make_plan(commType, dataType, tiling, d, transA, transB, p)) return;
+    if (!a || !b || !c) { fail(E_NULL, "a, b and c must be non-NULL"); return; }
+    if (commType == ALLGATHER_MATMUL) p.args.a[d->rankIdx] = a;
+    else p.args.a[0] = a;
+    p.args.b = b;
+    p.args.d = c;
+    if (!check_ptr_align(p, a, b)) p.variant = 0;
+    const int e = launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
+    if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
+    ok();
+}
+
+void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias,
+                  uint8_t *c_accum, uint8_t *d_out, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA,
+                  uint32_t transB, uint32_t outDataType)
+{
+    Plan p;
+    const CatcocSymmetricDesc *d = (const CatcocSymmetricDesc *)symmetricPtr;
+    if (make_plan(QUANT_MATMUL_REDUCE_SCATTER, INT8, tiling, d, transA, transB, p)) return;
+    if (!x1 || !x2 || !scale_x1 || !scale_x2 || !d_out) { fail(E_NULL, "x1, x2, scale_x1, scale_x2 and d_out must be non-NULL"); return; }
+    if (outDataType != FP16 && outDataType != BF16) { fail(E_DTYPE, "outDataType %u must be FP16 (1) or BF16 (27)", outDataType); return; }
+    p.args.a[0] = x1;
+    p.args.b = x2;
+    p.args.d = d_out;
+    p.args.scaleM = (const float *)scale_x1;
+    p.args.scaleN = (const float *)scale_x2;
+    p.args.bias = (const int32_t *)bias;
+    p.args.cAccum = (int32_t *)c_accum;
+    p.args.outDtype = outDataType;
+    if (!check_ptr_align(p, x1, x2) || (uintptr_t)scale_x2 % 16 != 0 || (bias && (uintptr_t)bias % 16 != 0) ||
+        (c_accum && (uintptr_t)c_accum % 16 != 0) || (uintptr_t)d_out % 8 != 0)
+        p.variant = 0;
+    const int e = launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
+    if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
+    ok();
+}
+
+}  // namespace
+
+extern "C" {
+
+#define FLOAT_LAUNCHER(name, commType, dataType)                                                                      \
+    void name(void *stream, uint64_t fftsAddr, uint8_t *a, uint8_t *b, uint8_t *c, uint8_t *aW, uint8_t *bW,           \
+              uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA, uint32_t transB)                        \
+    {                                                                                                                  \
+        (void)fftsAddr; (void)aW; (void)bW;                                                                            \
+        launch_float(commType, dataType, stream, a, b, c, symmetricPtr, tiling, transA, transB);                       \
+    }
+
+FLOAT_LAUNCHER(catcoc_launch_matmul_allreduce_fp16, MATMUL_ALLREDUCE, FP16)
+FLOAT_LAUNCHER(catcoc_launch_matmul_allreduce_bf16, MATMUL_ALLREDUCE, BF16)
+FLOAT_LAUNCHER(catcoc_launch_allgather_matmul_fp16, ALLGATHER_MATMUL, FP16)
+FLOAT_LAUNCHER(catcoc_launch_allgather_matmul_bf16, ALLGATHER_MATMUL, BF16)
+FLOAT_LAUNCHER(catcoc_launch_matmul_reduce_scatter_fp16, MATMUL_REDUCE_SCATTER, FP16)
+FLOAT_LAUNCHER(catcoc_launch_matmul_reduce_scatter_bf16, MATMUL_REDUCE_SCATTER, BF16)
+
+CatcocKernelFuncPtr catcoc_get_kernel(int commType, int dataType)
+{
+    switch ((commType << 8) | dataType) {  // key of KernelDispatcher::Hash, launch_map.h:30-33
+        case (MATMUL_ALLREDUCE << 8) | FP16: return catcoc_launch_matmul_allreduce_fp16;
+        case (MATMUL_ALLREDUCE << 8) | BF16: return catcoc_launch_matmul_allreduce_bf16;
+        case (ALLGATHER_MATMUL << 8) | FP16: return catcoc_launch_allgather_matmul_fp16;
+        case (ALLGATHER_MATMUL << 8) | BF16: return catcoc_launch_allgather_matmul_bf16;
+        case (MATMUL_REDUCE_SCATTER << 8) | FP16: return catcoc_launch_matmul_reduce_scatter_fp16;
+        case (MATMUL_REDUCE_SCATTER << 8) | BF16: return catcoc_launch_matmul_reduce_scatter_bf16;
+        default: return nullptr;
+    }
+}
+
+void catcoc_launch_quant_matmul_reduce_scatter(void *stream, uint64_t fftsAddr, uint8_t *x1, uint8_t *x2,
+                                               uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum,
+                                               uint8_t *d_out, uint8_t *symmetricPtr, CocTilingParams *tiling,
+                                               uint32_t transA, uint32_t transB, uint32_t outDataType)
+{
+    (void)fftsAddr;
+    launch_quant(stream, x1, x2, scale_x1, scale_x2, bias, c_accum, d_out, symmetricPtr, tiling, transA, transB, outDataType);
+}
+
+void catcoc_quant_matmul_reduce_scatter(void *stream, uint64_t fftsAddr, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1,
+                                        uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum, uint8_t *d_out,
+                                        uint8_t *symmetricPtr, uint32_t m, uint32_t n, uint32_t k)
+{
+    (void)fftsAddr;
+    // the example's fixed configuration (quant_matmul_reduce_scatter.cpp:93-147): tile 128x256, commInterval 10
+    CocTilingParams t;
+    memset(&t, 0, sizeof(t));
+    t.m = m; t.n = n; t.k = k;
+    t.m0 = 128; t.n0 = 256; t.k0 = 256;
+    t.commInterval = 10;
+    t.commTileM = 64; t.commBlockM = 64; t.commNpuSplit = 1; t.commDataSplit = 20;
+    const CatcocSymmetricDesc *d = (const CatcocSymmetricDesc *)symmetricPtr;
+    t.rankSize = (d && d->magic == CATCOC_DESC_MAGIC) ? d->rankSize : 0;
+    launch_quant(stream, x1, x2, scale_x1, scale_x2, bias, c_accum, d_out, symmetricPtr, &t, 0, 0, BF16);
+}
+
+const char *catcoc_last_error(void) { return g_err; }
+int catcoc_last_status(void) { return g_status; }
+
+int catcoc_can_implement(int commType, int dataType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
+                         uint32_t transA, uint32_t transB)
+{
+    Plan p;
+    const int e = make_plan(commType, dataType, tiling, desc, transA, transB, p);
+    if (!e) ok();
+    return e;
+}
+
+uint64_t catcoc_get_workspace_size(int commType, int dataType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc)
+{
+    Plan p;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
+    d = *desc;
+    d.flags &= ~CATCOC_OUTBOUND_MASK;  // size query must not require the buffer it sizes
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    if (make_plan(commType, dataType, tiling, &d, 0, 0, p)) return 0;
+    ok();
+    return (uint64_t)p.args.sched.stages * p.args.sched.blockPerComm * p.args.sched.m0 * p.args.sched.n0 * 4u;
+}
+
+uint32_t catcoc_get_task_count(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc)
+{
+    Plan p;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
+    d = *desc;
+    d.flags &= ~CATCOC_OUTBOUND_MASK;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    const int dataType = commType == QUANT_MATMUL_REDUCE_SCATTER ? INT8 : FP16;
+    if (make_plan(commType, dataType, tiling, &d, 0, 0, p)) return 0;
+    ok();
+    return p.args.sched.coreLoops;
+}
+
+int catcoc_task_tile(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t task,
+                     uint32_t *targetRank, uint32_t *row, uint32_t *col, uint32_t *wsRow)
+{
+    Plan p;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
+    d = *desc;
+    d.flags &= ~CATCOC_OUTBOUND_MASK;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    const int dataType = commType == QUANT_MATMUL_REDUCE_SCATTER ? INT8 : FP16;
+    if (make_plan(commType, dataType, tiling, &d, 0, 0, p)) return 0;
+    ok();
+    TileInfo ti;
+    if (!task_tile(p.args.sched, task, ti)) return 0;
+    if (targetRank) *targetRank = ti.targetRank;
+    if (row) *row = ti.row;
+    if (col) *col = ti.col;
+    if (wsRow) *wsRow = ti.wsRow;
+    return 1;
+}
+
+uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags)
+{
+    return workgroup_task(wg, tasks, (flags & CATCOC_FLAG_LINEAR_ORDER) != 0);
+}
+
+// ---- dynamic_tiling host logic ------------------------------------------------
+
+int catcoc_check_comm_interval_reduce_scatter(const CocTilingParams *t, int rankSize, int blockNum)
+{
+    return rankSize > 0 && ((int64_t)blockNum * t->commInterval) % rankSize == 0;
+}
+
+static int32_t max_peer_mem_per_rank(int rankSize)
+{
+    // (LCAL_BUFF_BYTES - FLAG_BUFF_BYTES) / INPUT_DTYPE / rankSize / MAX_BLOCK_COUNT, info.h:24-27
+    return (204 * 1024 * 1024 - 5 * 512 * 1024) / 2 / rankSize / 2;
+}
+
+int catcoc_check_comm_interval_allreduce(const CocTilingParams *t, int rankSize, int blockNum)
+{
+    if (rankSize <= 0) return 0;
+    return t->commInterval * t->m0 * t->n0 * (uint32_t)blockNum < (uint32_t)max_peer_mem_per_rank(rankSize);
+}
+
+int catcoc_check_comm_interval_allgather(const CocTilingParams *t, int rankSize)
+{
+    if (rankSize <= 0) return 0;
+    const uint32_t kLoop = t->k0 ? ceil_div(t->k, t->k0) : 0u;
+    return t->commInterval * t->m0 * t->k0 * kLoop < (uint32_t)max_peer_mem_per_rank(rankSize);
+}
+
+int catcoc_get_tilings(const CocTilingParams *base, int commType, int rankSize, int blockNum, CocTilingParams *out, int maxOut)
+{
+    // search space of tiling.h:19-22 in its nesting order: interval (outer), tile M, then the split pairs
+    static const uint32_t intervals[] = {4, 6, 8, 12, 14};
+    static const uint32_t tileMs[] = {4, 8, 16, 32, 64};
+    static const uint32_t splits[][2] = {{1, 16}, {1, 20}};
+    if (base == nullptr) { fail(E_NULL, "base tiling is NULL"); return 0; }
+    int n = 0;
+    for (uint32_t ci : intervals)
+        for (uint32_t tm : tileMs)
+            for (auto &sp : splits) {
+                CocTilingParams t = *base;
+                t.commInterval = ci;
+                t.commTileM = tm;
+                t.commBlockM = tm;
+                t.commNpuSplit = sp[0];
+                t.commDataSplit = sp[1];
+                bool valid = true;
+                if (commType == ALLGATHER_MATMUL) valid = catcoc_check_comm_interval_allgather(&t, rankSize);
+                else if (commType == MATMUL_REDUCE_SCATTER || commType == QUANT_MATMUL_REDUCE_SCATTER)
+                    valid = catcoc_check_comm_interval_reduce_scatter(&t, rankSize, blockNum);
+                else if (commType == MATMUL_ALLREDUCE) valid = catcoc_check_comm_interval_allreduce(&t, rankSize, blockNum);
+                if (!valid) continue;
+                if (out && n < maxOut) out[n] = t;
+                ++n;
+            }
+    return n;
+}
+
+uint32_t catcoc_get_splitk_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t coreNum, uint32_t m0, uint32_t n0, uint32_t k0)
+{
+    if (!m0 || !n0 || !k0 || !coreNum) return 1;
+    return splitk_factor(m, n, k, coreNum, m0, n0, k0);
+}
+
+void catcoc_default_tiling(CocTilingParams *t, uint32_t m, uint32_t k, uint32_t n, uint32_t rankSize)
+{
+    t->m = m; t->k = k; t->n = n;
+    t->m0 = 128; t->k0 = 256; t->n0 = 256;
+    t->commTileM = 64;
+    t->commInterval = 20;
+    t->commNpuSplit = 1;
+    t->commDataSplit = 2;
+    t->commBlockM = 64;
+    t->rankSize = rankSize;
+}
+
+// ---- schedulers on the host ---------------------------------------------------
+
+void catcoc_swizzle_block_coord(uint32_t off, uint32_t dir, uint32_t loopsM, uint32_t loopsN, uint32_t task, uint32_t *mIdx, uint32_t *nIdx)
+{
+    swizzle_block_coord(off, dir, loopsM, loopsN, task, *mIdx, *nIdx);
+}
+
+void catcoc_splitk_block_coord(uint32_t off, uint32_t dir, uint32_t loopsM, uint32_t loopsN, uint32_t kTiles, uint32_t f,
+                               uint32_t task, uint32_t *mIdx, uint32_t *nIdx, uint32_t *kIdx, uint32_t *slice)
+{
+    splitk_block_coord(off, dir, loopsM, loopsN, kTiles, f, task, *mIdx, *nIdx, *kIdx, *slice);
+}
+
+uint32_t catcoc_splitk_actual_k(uint32_t K, uint32_t k0, uint32_t f, uint32_t slice) { return splitk_actual_k(K, k0, f, slice); }
+
+void catcoc_allgather_block_coord(uint32_t off, uint32_t dir, uint32_t P, uint32_t commInterval, uint32_t loopsMRank,
+                                  uint32_t loopsN, uint32_t task, uint32_t *mIdx, uint32_t *nIdx)
+{
+    allgather_block_coord(off, dir, P, commInterval, loopsMRank, loopsN, task, *mIdx, *nIdx);
+}
+
+void catcoc_comm_block_idx(uint32_t dir, uint32_t P, uint32_t splitRow, uint32_t splitCol, uint32_t dataLoopsInRank,
+                           uint32_t task, uint32_t *dataIdx, uint32_t *rankIdx)
+{
+    comm_block_idx(dir, P, splitRow, splitCol, dataLoopsInRank, task, *dataIdx, *rankIdx);
+}
+
+int catcoc_device_info(int *cuCount, int *clockMHz, char *name, int nameLen)
+{
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+        return fail(E_LAUNCH, "no HIP device");
+    if (cuCount) *cuCount = prop.multiProcessorCount;
+    if (clockMHz) *clockMHz = prop.clockRate / 1000;
+    if (name && nameLen > 0) { strncpy(name, prop.gcnArchName, nameLen - 1); name[nameLen - 1] = 0; }
+    ok();
+    return 0;
+}
+
+const char *catcoc_version(void) { return "catcoc-hip 0.1 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,43 @@
+// Kernel argument block shared by the fused GEMM kernels and the host launcher.
+#pragma once
+#include <stdint.h>
+
+#include "tile_sched.h"
+
+namespace catcoc {
+
+constexpr int kMaxRanks = 16;
+
+// Element type codes: the CocDataType values of the C ABI.
+enum : uint32_t { DT_F16 = 1, DT_I8 = 2, DT_BF16 = 27 };
+
+enum : uint32_t {
+    GF_OUTBOUND_STORE = 1u << 0,  // non-kept tiles are stored to `outbound` (else folded into `checksum`)
+    GF_REDUCE_INT32 = 1u << 1,    // W8A8: peers are int32 and are added before the dequant
+    GF_LINEAR_ORDER = 1u << 2,    // workgroup i runs task i
+};
+
+struct GemmArgs {
+    const void *a[kMaxRanks];      // A operand per rank (all-gather: the P shards; otherwise a[0])
+    const void *b;
+    void *d;                       // kept rows, 16-bit output [keptRows, N]
+    const void *peers[kMaxRanks];  // staged peer partials for the kept rows
+    const float *scaleM;           // W8A8 per-token scale, indexed by global A row
+    const float *scaleN;           // W8A8 per-channel scale
+    const int32_t *bias;           // W8A8 optional int32 bias[N]
+    int32_t *cAccum;               // W8A8 optional int32 [keptRows, N]
+    void *accDump;                 // optional full [M, N] local partial (int32 / fp32)
+    void *outbound;                // tile-linear workspace for non-kept tiles
+    void *checksum;                // per-task int64 (W8A8) / double (float) sums of non-kept tiles
+    int64_t lda, ldb, ldd;         // leading dimensions in elements
+    int64_t peerLd, peerRowOffset;
+    uint32_t M, N, K;              // M = rows of the local A operand
+    uint32_t nPeers;
+    uint32_t keptBegin, keptRows;  // global rows [keptBegin, keptBegin + keptRows) are reduced and written to d
+    uint32_t flags;                // GF_*
+    uint32_t outDtype;             // DT_F16 / DT_BF16
+    uint32_t transA, transB;
+    SchedParams sched;
+};
+
+}  // namespace catcoc

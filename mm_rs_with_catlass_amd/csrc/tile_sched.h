@@ -1,0 +1,232 @@
+// Tile schedulers of the fused GEMM path, as integer functions that compile for
+// both the host (C ABI, CPU tests) and the device (kernels).  Written from the
+// behaviour of the reference's schedulers, cited per function (paths relative to
+// the reference tree).
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define CATCOC_HD __host__ __device__ inline
+#else
+#define CATCOC_HD inline
+#endif
+
+namespace catcoc {
+
+CATCOC_HD uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1u) / b; }
+CATCOC_HD uint32_t umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
+
+// Walk a 2-D grid in bands of `width` lines along the banded axis: inside a band
+// the banded axis runs fastest; with `serpentine` the other axis runs backwards
+// on odd bands.  The last band may be narrower.
+CATCOC_HD void banded_walk(uint32_t width, uint32_t lenBanded, uint32_t lenOther, uint32_t idx, bool serpentine,
+                           uint32_t &posBanded, uint32_t &posOther)
+{
+    const uint32_t perBand = width * lenOther;
+    const uint32_t band = idx / perBand;
+    const uint32_t in = idx - band * perBand;
+    const uint32_t w = umin(width, lenBanded - band * width);
+    const uint32_t q = in / w;
+    posBanded = band * width + (in - q * w);
+    posOther = (serpentine && (band & 1u)) ? lenOther - 1u - q : q;
+}
+
+// GemmIdentityBlockSwizzle<off,dir>::GetBlockCoord
+// (3rdparty/catlass/include/catlass/gemm/block/block_swizzle.hpp:79-113).
+// dir 0 bands tile rows, dir 1 bands tile columns.
+CATCOC_HD void swizzle_block_coord(uint32_t off, uint32_t dir, uint32_t loopsM, uint32_t loopsN, uint32_t task,
+                                   uint32_t &mIdx, uint32_t &nIdx)
+{
+    const uint32_t inner = task % (loopsM * loopsN);
+    if (dir == 0) banded_walk(off, loopsM, loopsN, inner, true, mIdx, nIdx);
+    else banded_walk(off, loopsN, loopsM, inner, true, nIdx, mIdx);
+}
+
+// SplitkGemmIdentityBlockSwizzle (block_swizzle.hpp:151-158): first k tile of slice s.
+CATCOC_HD uint32_t splitk_first_ktile(uint32_t kTiles, uint32_t f, uint32_t s)
+{
+    const uint32_t base = kTiles / f, extra = kTiles % f;
+    return s * base + umin(s, extra);
+}
+
+// block_swizzle.hpp:160-165,179-216.
+CATCOC_HD void splitk_block_coord(uint32_t off, uint32_t dir, uint32_t loopsM, uint32_t loopsN, uint32_t kTiles,
+                                  uint32_t f, uint32_t task, uint32_t &mIdx, uint32_t &nIdx, uint32_t &kIdx,
+                                  uint32_t &slice)
+{
+    const uint32_t mn = loopsM * loopsN;
+    slice = (task % (mn * f)) / mn;
+    kIdx = splitk_first_ktile(kTiles, f, slice);
+    swizzle_block_coord(off, dir, loopsM, loopsN, task % mn, mIdx, nIdx);
+}
+
+// block_swizzle.hpp:220-235: k extent of a slice (the last slice takes what is left of K).
+CATCOC_HD uint32_t splitk_actual_k(uint32_t K, uint32_t k0, uint32_t f, uint32_t s)
+{
+    const uint32_t kTiles = ceil_div(K, k0);
+    if (s == f - 1u) return K - splitk_first_ktile(kTiles, f, s) * k0;
+    return (kTiles / f + (s < kTiles % f ? 1u : 0u)) * k0;
+}
+
+// GemmIdentityBlockSwizzleAllGather::GetBlockCoord
+// (include/catcoc/dgemm/block/block_swizzle_allgather.hpp:88-108): tiles of one comm
+// round (commInterval tile rows from every rank) are swizzled as one grid, then the
+// row index is re-based rank-major.
+CATCOC_HD void allgather_block_coord(uint32_t off, uint32_t dir, uint32_t P, uint32_t commInterval,
+                                     uint32_t loopsMRank, uint32_t loopsN, uint32_t task, uint32_t &mIdx,
+                                     uint32_t &nIdx)
+{
+    const uint32_t rowsPerRound = commInterval * P;
+    const uint32_t rowsAll = loopsMRank * P;
+    const uint32_t rounds = ceil_div(rowsAll, rowsPerRound);
+    const uint32_t round = task / (rowsPerRound * loopsN);
+    const uint32_t inRound = task - round * rowsPerRound * loopsN;
+    const uint32_t rowsHere = (round == rounds - 1u) ? rowsAll - round * rowsPerRound : rowsPerRound;
+    const uint32_t perRank = rowsHere / P;
+    uint32_t cm, cn;
+    swizzle_block_coord(off, dir, rowsHere, loopsN, inRound, cm, cn);
+    const uint32_t r = cm / perRank;
+    mIdx = r * loopsMRank + round * commInterval + (cm - r * perRank);
+    nIdx = cn;
+}
+
+// BlockCommSwizzle<dir,false>::GetBlockIdx
+// (include/catcoc/comm_epilogue/block/comm_block_swizzle.hpp:147-186).
+CATCOC_HD void comm_block_idx(uint32_t dir, uint32_t P, uint32_t splitRow, uint32_t splitCol,
+                              uint32_t dataLoopsInRank, uint32_t task, uint32_t &dataIdx, uint32_t &rankIdx)
+{
+    const uint32_t inner = task % (dataLoopsInRank * P);
+    uint32_t d, r;
+    if (dir == 0) banded_walk(splitRow, dataLoopsInRank, P, inner, false, d, r);
+    else banded_walk(splitCol, P, dataLoopsInRank, inner, false, r, d);
+    const uint32_t stepped = r * (P / splitCol);
+    r = (stepped % P + stepped / P + d) % P;
+    dataIdx = d;
+    rankIdx = r;
+}
+
+// ---------------------------------------------------------------------------
+// Task -> tile of each operator
+// ---------------------------------------------------------------------------
+
+enum : uint32_t { OP_ALLREDUCE = 0, OP_ALLGATHER = 1, OP_REDUCE_SCATTER = 2 };
+
+struct SchedParams {
+    uint32_t op;            // OP_*
+    uint32_t P;             // rankSize
+    uint32_t mRank;         // rows of one rank's sub-problem (RS: M/P, AG: shard rows, AR: M)
+    uint32_t N;
+    uint32_t m0, n0;
+    uint32_t loopsM, loopsN;  // tile grid of ONE rank's sub-problem
+    uint32_t coreLoops;       // tasks of the launch
+    uint32_t blockPerComm;    // blockNum * commInterval
+    uint32_t commInterval;
+    uint32_t stages;
+    uint32_t off, dir;
+};
+
+struct TileInfo {
+    uint32_t targetRank;  // rank whose row block the tile belongs to (AG: rank whose shard feeds it)
+    uint32_t rowInRank;   // first row inside that rank's sub-problem
+    uint32_t row;         // first row in the global problem
+    uint32_t col;         // first column
+    uint32_t rowsValid, colsValid;
+    uint32_t wsRow;       // first row of the tile in the reference's tile-linear workspace
+};
+
+CATCOC_HD SchedParams make_sched(uint32_t op, uint32_t M, uint32_t N, uint32_t P, uint32_t m0, uint32_t n0,
+                                 uint32_t blockNum, uint32_t commInterval, uint32_t stages, uint32_t off,
+                                 uint32_t dir)
+{
+    SchedParams s;
+    s.op = op;
+    s.P = P;
+    s.mRank = (op == OP_REDUCE_SCATTER) ? M / P : M;  // AG: M is already the shard's rows
+    s.N = N;
+    s.m0 = m0;
+    s.n0 = n0;
+    s.loopsM = ceil_div(s.mRank, m0);
+    s.loopsN = ceil_div(N, n0);
+    s.coreLoops = s.loopsM * s.loopsN * (op == OP_ALLREDUCE ? 1u : P);
+    s.blockPerComm = blockNum * commInterval;
+    s.commInterval = commInterval;
+    s.stages = stages;
+    s.off = off;
+    s.dir = dir;
+    return s;
+}
+
+// quant_matmul_reduce_scatter.hpp:159-201 / matmul_reduce_scatter.hpp (same mapping),
+// matmul_allreduce.hpp:146-179, allgather_matmul.hpp:131-163.
+CATCOC_HD bool task_tile(const SchedParams &s, uint32_t t, TileInfo &ti)
+{
+    if (t >= s.coreLoops) return false;
+    uint32_t mi, ni;
+    if (s.op == OP_REDUCE_SCATTER) {
+        const uint32_t perRank = s.blockPerComm / s.P;
+        const uint32_t commLoops = ceil_div(s.coreLoops, s.blockPerComm);
+        const uint32_t round = t / s.blockPerComm;
+        const uint32_t b = t - round * s.blockPerComm;
+        const uint32_t actual = (round == commLoops - 1u) ? s.coreLoops - round * s.blockPerComm : s.blockPerComm;
+        const uint32_t actualInRank = actual / s.P;
+        ti.targetRank = b / actualInRank;
+        swizzle_block_coord(s.off, s.dir, s.loopsM, s.loopsN, round * perRank + b % actualInRank, mi, ni);
+        ti.wsRow = ((round % s.stages) * s.blockPerComm + b) * s.m0;
+    } else if (s.op == OP_ALLREDUCE) {
+        const uint32_t round = t / s.blockPerComm;
+        ti.targetRank = 0;
+        swizzle_block_coord(s.off, s.dir, s.loopsM, s.loopsN, t, mi, ni);
+        ti.wsRow = ((round % s.stages) * s.blockPerComm + (t - round * s.blockPerComm)) * s.m0;
+    } else {
+        uint32_t mAll;
+        allgather_block_coord(s.off, s.dir, s.P, s.commInterval, s.loopsM, s.loopsN, t, mAll, ni);
+        ti.targetRank = mAll / s.loopsM;
+        mi = mAll - ti.targetRank * s.loopsM;
+        // workspace row of the A block in the reference (allgather_matmul.hpp:150-161):
+        // (stage * commInterval*P + rank * tileRowsPerRankThisRound + inCommIdx) * m0
+        const uint32_t round = mi / s.commInterval;
+        const uint32_t rounds = ceil_div(s.loopsM, s.commInterval);
+        const uint32_t perRank = (round == rounds - 1u) ? s.loopsM - round * s.commInterval : s.commInterval;
+        ti.wsRow = ((round % s.stages) * s.commInterval * s.P + ti.targetRank * perRank + mi % s.commInterval) * s.m0;
+    }
+    ti.rowInRank = mi * s.m0;
+    ti.row = ti.targetRank * s.mRank + ti.rowInRank;
+    ti.col = ni * s.n0;
+    ti.rowsValid = umin(s.m0, s.mRank - ti.rowInRank);
+    ti.colsValid = umin(s.n0, s.N - ti.col);
+    return true;
+}
+
+// Workgroup -> task.  Hardware deals consecutive workgroups round-robin over the 8
+// XCDs (each with its own L2); chunks of 16 consecutive tasks (neighbours in the
+// swizzle, sharing A rows and B columns) are dealt to one XCD each, and successive
+// chunks rotate over the XCDs so that every XCD gets the same share of each rank's
+// tiles, including the expensive kept ones.  A bijection on [0,tasks).
+CATCOC_HD uint32_t workgroup_task(uint32_t wg, uint32_t tasks, bool linear)
+{
+    const uint32_t X = 8u, CH = 16u;
+    const uint32_t full = tasks / (X * CH) * (X * CH);
+    if (linear || wg >= full) return wg;
+    const uint32_t x = wg % X, s = wg / X;
+    return ((s / CH) * X + x) * CH + s % CH;
+}
+
+// SplitkMatmul::GetSplitkFactor (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:219-265).
+inline uint32_t splitk_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t cores, uint32_t m0, uint32_t n0,
+                              uint32_t k0)
+{
+    const uint32_t cap = k <= 1024 ? 2u : k <= 2048 ? 4u : k <= 4096 ? 8u : 16u;
+    const uint32_t base = ceil_div(m, m0) * ceil_div(n, n0);
+    uint32_t f = umin(cores / base, cap);
+    if (f == 0) f = 1;
+    if (base < cores) {
+        // keep growing while one more slice does not cost an extra wave of tiles
+        while (f < cap && ceil_div(base * f, cores) >= ceil_div(base, cores) * f) ++f;
+    }
+    f = umin(f, ceil_div(k, k0));
+    if (k > 8192 && f < 2) f = 2;
+    if (k > 32768 && f < 4) f = 4;
+    return f;
+}
+
+}  // namespace catcoc

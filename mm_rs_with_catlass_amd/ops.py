@@ -1,0 +1,159 @@
+"""Host-side mirror of the reference's operator entry points, on torch tensors resident in HBM.
+
+Each function fills the reference's ``CocTilingParams`` and the one-GPU symmetric
+descriptor, then calls the matching C-ABI launcher of ``libcatcoc_hip.so``
+(``include/catcoc_hip.h``) on torch's current stream.  torch is used for device
+memory and streams only; all arithmetic happens in the HIP kernels.
+
+Reference entry points mirrored (paths relative to the reference tree):
+  ShmemQuantMatmulReduceScatter   examples/02_matmul_reduce_scatter/quant_matmul_reduce_scatter.cpp:54-60
+  LaunchMatmulReduceScatter*      examples/dynamic_tiling/impl/kernel_fp16.cpp:64-86
+  LaunchMatmulAllReduce*          examples/dynamic_tiling/impl/kernel_fp16.cpp:22-44
+  LaunchAllGatherMatmul*          examples/dynamic_tiling/impl/kernel_fp16.cpp:46-62
+"""
+import ctypes as C
+
+import torch
+
+from . import lib as _l
+
+_TORCH_TO_DT = {torch.float16: _l.FP16, torch.bfloat16: _l.BF16}
+
+
+def default_tiling(m, k, n, rank_size, **over):
+    """The defaults of examples/dynamic_tiling/dynamic_tiling.cpp:215-227, with overrides.
+    m0/n0/k0 = 0 lets the library pick its own macro tile."""
+    t = _l.CocTilingParams()
+    _l.load().catcoc_default_tiling(C.byref(t), m, k, n, rank_size)
+    t.commInterval = 1
+    for key, val in over.items():
+        setattr(t, key, val)
+    return t
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _check_dev(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise _l.CatcocError("all operands must live on the GPU (got a %s tensor)" % t.device)
+        if t is not None and not t.is_contiguous():
+            raise _l.CatcocError("operands must be contiguous")
+
+
+def _desc(rank, rank_size, peers, peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump):
+    peer_ld = peers[0].shape[1] if peers else 0
+    return _l.make_desc(
+        rank, rank_size, [p.data_ptr() for p in peers], peer_ld, peer_row_offset, flags, block_num, stages, swizzle,
+        _ptr(outbound), outbound.numel() * outbound.element_size() if outbound is not None else 0,
+        _ptr(checksum), _ptr(acc_dump))
+
+
+def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(), rank=0, rank_size=1,
+                                        out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
+                                        reduce_int32=False, outbound=None, checksum=None, acc_dump=None,
+                                        c_accum=None, block_num=0, stages=0, swizzle=None, linear_order=False,
+                                        out=None):
+    """Validate and bind the arguments once; returns (launch, out) where launch() enqueues one call of
+    catcoc_launch_quant_matmul_reduce_scatter on torch's current stream (for launch-rate-sensitive loops)."""
+    _check_dev(x1, x2, scale_x1, scale_x2, bias, outbound, checksum, acc_dump, c_accum, *peers)
+    m, k = x1.shape
+    n = x2.shape[0] if trans_b else x2.shape[1]
+    t = tiling if tiling is not None else default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
+    flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_REDUCE_INT32 if reduce_int32 else 0) | \
+        (_l.FLAG_LINEAR_ORDER if linear_order else 0)
+    d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
+    if out is None:
+        out = torch.empty((m // max(rank_size, 1), n), dtype=out_dtype, device=x1.device)
+    L = _l.load()
+    keep = (x1, x2, scale_x1, scale_x2, bias, tuple(peers), outbound, checksum, acc_dump, c_accum, out, d, t)
+    fn = L.catcoc_launch_quant_matmul_reduce_scatter
+    argv = (0, x1.data_ptr(), x2.data_ptr(), scale_x1.data_ptr(), scale_x2.data_ptr(), _ptr(bias), _ptr(c_accum),
+            out.data_ptr(), C.addressof(d), C.byref(t), 0, int(trans_b), _TORCH_TO_DT[out.dtype])
+
+    def launch(_keep=keep):
+        fn(_stream(), *argv)
+
+    return launch, out
+
+
+def quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(), rank=0, rank_size=1,
+                                out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
+                                reduce_int32=False, outbound=None, checksum=None, acc_dump=None, c_accum=None,
+                                block_num=0, stages=0, swizzle=None, linear_order=False, out=None):
+    """W8A8 matmul -> reduce-scatter share of one rank.
+
+    x1 [m,k] int8, x2 [k,n] int8 ([n,k] with trans_b), scale_x1 [m] fp32 per token, scale_x2 [n] fp32 per
+    channel, bias [n] int32 or None.  peers: rank_size-1 staged partials for the kept rows (fp32, or int32
+    with reduce_int32), added in list order after the local partial.  Returns d_out [m/rank_size, n].
+    """
+    launch, out = prepare_quant_matmul_reduce_scatter(
+        x1, x2, scale_x1, scale_x2, bias, peers, rank, rank_size, out_dtype, tiling, trans_b, peer_row_offset,
+        reduce_int32, outbound, checksum, acc_dump, c_accum, block_num, stages, swizzle, linear_order, out)
+    launch()
+    _l.check()
+    return out
+
+
+def _float_op(comm_type, a, b, c_shape, peers, rank, rank_size, tiling, trans_a, trans_b, peer_row_offset, outbound,
+              checksum, acc_dump, block_num, stages, swizzle, linear_order, out, m_for_tiling):
+    _check_dev(a, b, outbound, checksum, acc_dump, *peers)
+    if a.dtype not in _TORCH_TO_DT or b.dtype != a.dtype:
+        raise _l.CatcocError("a and b must both be float16 or both bfloat16")
+    k = a.shape[0] if trans_a else a.shape[1]
+    n = b.shape[0] if trans_b else b.shape[1]
+    t = tiling if tiling is not None else default_tiling(m_for_tiling, k, n, rank_size, m0=0, n0=0, k0=0)
+    flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_LINEAR_ORDER if linear_order else 0)
+    d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
+    if out is None:
+        out = torch.empty(c_shape(n), dtype=a.dtype, device=a.device)
+    L = _l.load()
+    fn = L.catcoc_get_kernel(comm_type, _TORCH_TO_DT[a.dtype])
+    if not fn:
+        raise _l.CatcocError("no kernel registered for commType %d dtype %s" % (comm_type, a.dtype))
+    _l.KernelFuncPtr(fn)(_stream(), 0, a.data_ptr(), b.data_ptr(), out.data_ptr(), None, None, C.addressof(d),
+                         C.byref(t), int(trans_a), int(trans_b))
+    _l.check()
+    return out
+
+
+def matmul_reduce_scatter(a, b, peers=(), rank=0, rank_size=1, tiling=None, trans_a=False, trans_b=False,
+                          peer_row_offset=0, outbound=None, checksum=None, acc_dump=None, block_num=0, stages=0,
+                          swizzle=None, linear_order=False, out=None):
+    """fp16/bf16 matmul -> reduce-scatter share: a [m,k], b [k,n], peers fp32; returns [m/rank_size, n]."""
+    m = a.shape[1] if trans_a else a.shape[0]
+    return _float_op(_l.MATMUL_REDUCE_SCATTER, a, b, lambda n: (m // max(rank_size, 1), n), peers, rank, rank_size,
+                     tiling, trans_a, trans_b, peer_row_offset, outbound, checksum, acc_dump, block_num, stages,
+                     swizzle, linear_order, out, m)
+
+
+def matmul_allreduce(a, b, peers=(), rank=0, rank_size=1, tiling=None, trans_a=False, trans_b=False,
+                     peer_row_offset=0, acc_dump=None, block_num=0, stages=0, swizzle=None, linear_order=False,
+                     out=None):
+    """fp16/bf16 matmul -> all-reduce share: every row is kept; peers are full [m,n] fp32 partials."""
+    m = a.shape[1] if trans_a else a.shape[0]
+    return _float_op(_l.MATMUL_ALLREDUCE, a, b, lambda n: (m, n), peers, rank, rank_size, tiling, trans_a, trans_b,
+                     peer_row_offset, None, None, acc_dump, block_num, stages, swizzle, linear_order, out, m)
+
+
+def allgather_matmul(a_local, peer_shards, b, rank=0, rank_size=1, tiling=None, trans_b=False, acc_dump=None,
+                     block_num=0, stages=0, swizzle=None, linear_order=False, out=None):
+    """all-gather -> matmul: a_local [m,k] is this rank's shard, peer_shards the other ranks' shards in
+    ascending rank order (separate buffers, read in place); returns [m*rank_size, n]."""
+    m = a_local.shape[0]
+    return _float_op(_l.ALLGATHER_MATMUL, a_local, b, lambda n: (m * rank_size, n), peer_shards, rank, rank_size,
+                     tiling, False, trans_b, 0, None, None, acc_dump, block_num, stages, swizzle, linear_order, out, m)
+
+
+def device_info():
+    cu, mhz = C.c_int(), C.c_int()
+    name = C.create_string_buffer(64)
+    if _l.load().catcoc_device_info(C.byref(cu), C.byref(mhz), name, 64) != 0:
+        raise _l.CatcocError(_l.last_error())
+    return {"cu_count": cu.value, "clock_mhz": mhz.value, "arch": name.value.decode()}

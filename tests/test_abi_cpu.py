@@ -1,0 +1,202 @@
+"""CPU tests of the C-ABI library: exports, host-side scheduling and tiling logic (the same
+integer code the kernels run) against the oracle, and argument validation.  No kernel is launched."""
+import ctypes as C
+import re
+import os
+
+import pytest
+
+import oracle
+from mm_rs_with_catlass_amd import lib as L
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+u32 = C.c_uint32
+
+
+@pytest.fixture(scope="module")
+def so():
+    return L.load()
+
+
+def test_library_exports_every_declared_symbol(so):
+    hdr = open(os.path.join(ROOT, "include", "catcoc_hip.h")).read()
+    declared = set(re.findall(r"\b(catcoc_[a-z0-9_]+)\s*\(", hdr))
+    assert declared, "no declarations found"
+    assert declared == set(L.EXPORTS)
+    for name in declared:
+        assert hasattr(so, name), name
+
+
+def test_struct_layout_matches_reference_tiling_params():
+    # twelve uint32 in the reference's order (examples/dynamic_tiling/include/info.h:29-42)
+    names = [f[0] for f in L.CocTilingParams._fields_]
+    assert names == ["m", "k", "n", "m0", "k0", "n0", "commTileM", "commInterval", "commNpuSplit",
+                     "commDataSplit", "commBlockM", "rankSize"]
+    assert C.sizeof(L.CocTilingParams) == 48
+    assert [getattr(L.CocTilingParams, n).offset for n in names] == list(range(0, 48, 4))
+
+
+def test_registry_matches_reference_dispatcher(so):
+    # launch_map.h:60-66 registers the three ops for FP16 and BF16; anything else is NULL
+    for ct in (L.MATMUL_ALLREDUCE, L.ALLGATHER_MATMUL, L.MATMUL_REDUCE_SCATTER):
+        for dt in (L.FP16, L.BF16):
+            assert so.catcoc_get_kernel(ct, dt)
+        assert not so.catcoc_get_kernel(ct, 0)
+        assert not so.catcoc_get_kernel(ct, L.INT8)
+    assert not so.catcoc_get_kernel(7, L.FP16)
+    names = {(L.MATMUL_ALLREDUCE, L.FP16): "catcoc_launch_matmul_allreduce_fp16",
+             (L.ALLGATHER_MATMUL, L.BF16): "catcoc_launch_allgather_matmul_bf16",
+             (L.MATMUL_REDUCE_SCATTER, L.BF16): "catcoc_launch_matmul_reduce_scatter_bf16"}
+    for (ct, dt), nm in names.items():
+        assert so.catcoc_get_kernel(ct, dt) == C.cast(getattr(so, nm), C.c_void_p).value
+
+
+def test_host_schedulers_equal_oracle(so):
+    m, n, k, s = u32(), u32(), u32(), u32()
+    for off, d, lm, ln in [(7, 1, 8, 16), (7, 1, 4, 16), (7, 0, 16, 4), (3, 0, 11, 3), (3, 1, 11, 9), (1, 0, 3, 2),
+                           (2, 1, 5, 5), (4, 0, 1, 1), (7, 1, 1, 32)]:
+        for t in range(2 * lm * ln):
+            so.catcoc_swizzle_block_coord(off, d, lm, ln, t, C.byref(m), C.byref(n))
+            assert (m.value, n.value) == oracle.swizzle_block_coord(off, d, lm, ln, t)
+    for off, d, lm, ln, kt, f in [(7, 1, 1, 32, 32, 8), (3, 0, 4, 32, 32, 2), (3, 0, 1, 3, 8, 3), (1, 1, 1, 2, 9, 4),
+                                  (7, 1, 1, 4, 8, 5)]:
+        for t in range(lm * ln * f):
+            so.catcoc_splitk_block_coord(off, d, lm, ln, kt, f, t, C.byref(m), C.byref(n), C.byref(k), C.byref(s))
+            assert (m.value, n.value, k.value, s.value) == oracle.splitk_block_coord(off, d, lm, ln, kt, f, t)
+        for sl in range(f):
+            for K in (kt * 256, kt * 256 - 100):
+                assert so.catcoc_splitk_actual_k(K, 256, f, sl) == oracle.splitk_actual_k(K, 256, f, sl)
+    for off, d, P, ci, lmr, ln in [(7, 1, 8, 1, 4, 4), (7, 1, 8, 3, 4, 4), (7, 1, 2, 2, 6, 3), (3, 0, 4, 2, 5, 4)]:
+        for t in range(lmr * P * ln):
+            so.catcoc_allgather_block_coord(off, d, P, ci, lmr, ln, t, C.byref(m), C.byref(n))
+            assert (m.value, n.value) == oracle.allgather_block_coord(off, d, P, ci, lmr, ln, t)
+    for d, P, sr, sc, dl in [(0, 8, 20, 1, 50), (0, 8, 16, 1, 7), (0, 4, 2, 2, 9), (1, 8, 4, 2, 13), (1, 2, 3, 1, 5)]:
+        for t in range(dl * P + 5):
+            so.catcoc_comm_block_idx(d, P, sr, sc, dl, t, C.byref(m), C.byref(n))
+            assert (m.value, n.value) == oracle.comm_block_idx(d, P, sr, sc, dl, t)
+
+
+def _desc(P, rank=0, **kw):
+    return L.make_desc(rank, P, [16] * (P - 1), **kw)
+
+
+def test_task_tile_equals_oracle_reduce_scatter_and_allreduce(so):
+    tr, row, col, ws = u32(), u32(), u32(), u32()
+    for (M, N, P, m0, n0, bn, ci, st) in [(8192, 4096, 8, 128, 256, 20, 10, 2), (8192, 4096, 8, 128, 256, 256, 1, 2),
+                                          (4096, 4096, 8, 128, 256, 256, 4, 2), (800, 260, 8, 64, 256, 16, 1, 3)]:
+        t = L.CocTilingParams(m=M, k=64, n=N, m0=m0, n0=n0, k0=256, commInterval=ci, rankSize=P)
+        d = _desc(P, block_num=bn, stages=st)
+        cnt = so.catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+        assert cnt == -(-(M // P) // m0) * -(-N // n0) * P
+        for task in list(range(0, cnt, max(1, cnt // 97))) + [cnt - 1]:
+            assert so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr),
+                                       C.byref(row), C.byref(col), C.byref(ws))
+            o = oracle.rs_task(M, N, P, m0, n0, bn, ci, st, task)
+            assert (tr.value, row.value, col.value, ws.value) == (o[0], o[3], o[4], o[5])
+        assert not so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), cnt, C.byref(tr),
+                                       C.byref(row), C.byref(col), C.byref(ws))
+    t = L.CocTilingParams(m=512, k=2048, n=1024, m0=128, n0=256, k0=256, commInterval=3, rankSize=2)
+    d = _desc(2, block_num=20)
+    for task in range(16):
+        assert so.catcoc_task_tile(L.MATMUL_ALLREDUCE, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row),
+                                   C.byref(col), C.byref(ws))
+        mi, ni, w = oracle.ar_task(512, 1024, 128, 256, 20, 3, 2, task)
+        assert (row.value, col.value, ws.value) == (mi * 128, ni * 256, w)
+
+
+def test_workgroup_task_is_a_bijection(so):
+    for tasks in (1, 7, 127, 128, 129, 1024, 1000, 2048, 4097):
+        for flags in (0, L.FLAG_LINEAR_ORDER):
+            got = sorted(so.catcoc_workgroup_task(w, tasks, flags) for w in range(tasks))
+            assert got == list(range(tasks))
+    # chunks of 16 consecutive tasks share an XCD (workgroup id modulo 8)
+    xcd = {}
+    for w in range(1024):
+        xcd.setdefault(so.catcoc_workgroup_task(w, 1024, 0) // 16, set()).add(w % 8)
+    assert all(len(v) == 1 for v in xcd.values())
+    # every XCD gets the same number of each rank's 128 tasks
+    for r in range(8):
+        per = [0] * 8
+        for w in range(1024):
+            if so.catcoc_workgroup_task(w, 1024, 0) // 128 == r:
+                per[w % 8] += 1
+        assert per == [16] * 8
+
+
+def test_tiling_search_equals_oracle(so):
+    for ct, octx in ((L.MATMUL_ALLREDUCE, oracle.MATMUL_ALLREDUCE), (L.ALLGATHER_MATMUL, oracle.ALLGATHER_MATMUL),
+                     (L.MATMUL_REDUCE_SCATTER, oracle.MATMUL_REDUCE_SCATTER)):
+        for P in (2, 3, 8):
+            for (m, k, n) in ((8192, 1792, 4096), (8192, 27392, 4096), (7936, 12544, 6656)):
+                base = L.CocTilingParams()
+                so.catcoc_default_tiling(C.byref(base), m, k, n, P)
+                assert (base.m0, base.k0, base.n0, base.commTileM, base.commInterval, base.commNpuSplit,
+                        base.commDataSplit, base.commBlockM) == (128, 256, 256, 64, 20, 1, 2, 64)
+                out = (L.CocTilingParams * 64)()
+                cnt = so.catcoc_get_tilings(C.byref(base), ct, P, 20, out, 64)
+                ob = oracle.TilingParams(*[getattr(base, f[0]) for f in L.CocTilingParams._fields_])
+                want = oracle.get_tilings(ob, octx, P, 20)
+                assert cnt == len(want)
+                for i in range(cnt):
+                    for f, _ in L.CocTilingParams._fields_:
+                        assert getattr(out[i], f) == getattr(want[i], f)
+
+
+def test_splitk_factor_equals_oracle(so):
+    for (m, n, k, cores) in [(16, 8192, 8192, 20), (16, 8192, 8192, 256), (512, 8192, 8192, 256), (128, 256, 1024, 20),
+                             (128, 256, 256, 20), (4096, 4096, 9000, 20), (4096, 4096, 40000, 20), (768, 256, 4096, 20),
+                             (1, 8192, 8192, 256), (64, 8192, 8192, 256), (128, 8192, 8192, 256)]:
+        assert so.catcoc_get_splitk_factor(m, n, k, cores, 128, 256, 256) == oracle.splitk_factor(m, n, k, cores, 128, 256, 256)
+
+
+def test_validation_errors(so):
+    t = L.CocTilingParams(m=1024, k=256, n=512, rankSize=8, commInterval=1)
+    d = _desc(8)
+    chk = lambda ct, dt, tt, dd, ta=0, tb=0: so.catcoc_can_implement(ct, dt, C.byref(tt) if tt else None,
+                                                                     C.byref(dd) if dd else None, ta, tb)
+    assert chk(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, t, d) == 0 and L.last_error() == ""
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t, d) == 0
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, None, d) != 0 and "NULL" in L.last_error()
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t, None) != 0
+    bad = _desc(8); bad.magic = 0
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t, bad) != 0 and "magic" in L.last_error()
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.INT8, t, d) != 0          # int8 is only registered for the quant op
+    assert chk(L.QUANT_MATMUL_REDUCE_SCATTER, L.FP16, t, d) != 0
+    t2 = L.CocTilingParams(m=1001, k=256, n=512, rankSize=8, commInterval=1)
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t2, d) != 0 and "rankSize" in L.last_error()   # m % P != 0
+    t3 = L.CocTilingParams(m=1024, k=256, n=512, rankSize=4, commInterval=1)
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t3, d) != 0          # tiling and descriptor disagree on rankSize
+    d3 = _desc(3, block_num=20)
+    t4 = L.CocTilingParams(m=3 * 128, k=256, n=512, rankSize=3, commInterval=4)
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t4, d3) != 0 and "multiple of rankSize" in L.last_error()  # 80 % 3
+    t4.commInterval = 6
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t4, d3) == 0
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, L.CocTilingParams(m=0, k=1, n=1), d) != 0     # empty problem
+    dnp = L.make_desc(0, 8, [16] * 3)
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t, dnp) != 0 and "peers[3]" in L.last_error()   # missing peer
+    dr = L.make_desc(9, 8, [16] * 7)
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t, dr) != 0
+    dst = L.make_desc(0, 8, [16] * 7, flags=L.OUTBOUND_STORE)
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t, dst) != 0 and "outbound" in L.last_error()
+    need = so.catcoc_get_workspace_size(L.MATMUL_REDUCE_SCATTER, L.FP16, C.byref(t), C.byref(dst))
+    assert need == 2 * 256 * 128 * 256 * 4
+    dst.outbound, dst.outboundBytes = 4096, need - 1
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t, dst) != 0 and "too small" in L.last_error()
+    dst.outboundBytes = need
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t, dst) == 0
+    dri = L.make_desc(0, 8, [16] * 7, flags=L.FLAG_REDUCE_INT32)
+    assert chk(L.MATMUL_REDUCE_SCATTER, L.FP16, t, dri) != 0        # int32 reduce is a W8A8 mode
+    assert chk(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, t, dri) == 0
+
+
+def test_rejected_launch_launches_nothing_and_reports(so):
+    # a launcher called with a bad descriptor must return without touching the GPU
+    t = L.CocTilingParams(m=1024, k=256, n=512, rankSize=8, commInterval=1)
+    bad = L.make_desc(0, 8, [16] * 7); bad.magic = 1
+    so.catcoc_launch_matmul_reduce_scatter_fp16(None, 0, 16, 16, 16, None, None, C.addressof(bad), C.byref(t), 0, 0)
+    assert so.catcoc_last_status() != 0 and "magic" in L.last_error()
+    with pytest.raises(L.CatcocError):
+        L.check()
+    so.catcoc_quant_matmul_reduce_scatter(None, 0, 16, 16, 16, 16, None, None, 16, None, 1024, 512, 256)
+    assert so.catcoc_last_status() != 0

@@ -1,0 +1,338 @@
+"""GPU parity tests: the HIP library, called through its C ABI, against the CPU oracle on the same
+seeded inputs.  Bars: int32 accumulators bit-exact; W8A8 outputs within 1 ulp of the 16-bit output
+type (the build reduces in the oracle's order, so they are normally equal); float GEMMs within
+rel-err 1e-2 of the fp32 k-sequential oracle and inside the reference's own rtol gate."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from mm_rs_with_catlass_amd import lib as L
+from mm_rs_with_catlass_amd import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU test selected but no GPU is visible")
+    L.load()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def dev16(bits, dtype):
+    """uint16 bit patterns -> fp16 / bf16 tensor on the GPU."""
+    t = torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).to(DEV)
+    return t.view(torch.float16 if dtype == oracle.FP16 else torch.bfloat16)
+
+
+def host16(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def ulp_diff16(a_bits, b_bits):
+    """Distance in units of last place between two arrays of fp16/bf16 bit patterns."""
+    def key(x):
+        x = x.astype(np.int32)
+        return np.where(x & 0x8000, -(x & 0x7FFF), x & 0x7FFF)
+    return np.abs(key(a_bits) - key(b_bits))
+
+
+TORCH_DT = {oracle.FP16: torch.float16, oracle.BF16: torch.bfloat16}
+
+
+def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, trans_b=False, reduce_int32=False,
+               full_peers=False, tiling=None, outbound=False, block_num=0, stages=0, swizzle=None, linear=False):
+    _need_gpu()
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.integers(-1000, 1000, N, dtype=np.int32) if bias else None
+    rows = M // P
+    prow0 = rank * rows if full_peers else 0
+    prow = M if full_peers else rows
+    if reduce_int32:
+        peers = [rng.integers(-2 ** 24, 2 ** 24, (prow, N), dtype=np.int32) for _ in range(P - 1)]
+    else:
+        peers = [rng.standard_normal((prow, N)).astype(np.float32) for _ in range(P - 1)]
+    acc_want, out_want = oracle.quant_matmul_reduce_scatter(
+        x1, x2, s1, s2, b, rank * rows, rows, peers, out_dtype, peer_row0=prow0, reduce_int32=reduce_int32)
+
+    x2d = dev(np.ascontiguousarray(x2.T)) if trans_b else dev(x2)
+    acc_dump = torch.full((M, N), -7, dtype=torch.int32, device=DEV)
+    c_accum = torch.full((rows, N), -7, dtype=torch.int32, device=DEV)
+    dpeers = [dev(p) for p in peers]
+    import ctypes as C
+    kw = {}
+    ob = None
+    t = tiling if tiling is not None else ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+    d = L.make_desc(rank, P, [16] * (P - 1), block_num=block_num, stages=stages, swizzle=swizzle)
+    ntasks = L.load().catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+    if outbound:
+        need = L.load().catcoc_get_workspace_size(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, C.byref(t), C.byref(d))
+        ob = torch.zeros(need // 4, dtype=torch.int32 if reduce_int32 else torch.float32, device=DEV)
+        kw["outbound"] = ob
+    checksum = torch.zeros(ntasks, dtype=torch.int64, device=DEV)
+    if not outbound:
+        kw["checksum"] = checksum
+    out = ops.quant_matmul_reduce_scatter(
+        dev(x1), x2d, dev(s1), dev(s2), dev(b) if bias else None, dpeers, rank, P, out_dtype=TORCH_DT[out_dtype],
+        tiling=tiling, trans_b=trans_b, peer_row_offset=prow0, reduce_int32=reduce_int32, acc_dump=acc_dump,
+        c_accum=c_accum, block_num=block_num, stages=stages, swizzle=swizzle, linear_order=linear, **kw)
+    torch.cuda.synchronize()
+    acc_got = acc_dump.cpu().numpy()
+    assert np.array_equal(acc_got, acc_want), "int32 accumulators differ from the oracle"
+    kept = acc_want[rank * rows:(rank + 1) * rows]
+    if reduce_int32:
+        kept = kept + sum(p[prow0:prow0 + rows] for p in peers)
+    assert np.array_equal(c_accum.cpu().numpy(), kept)
+    got = host16(out)
+    d_ulp = ulp_diff16(got, out_want)
+    assert d_ulp.max() <= 1, "output differs by %d ulp" % d_ulp.max()
+    return dict(x1=x1, x2=x2, s1=s1, s2=s2, bias=b, acc=acc_want, out=got, out_want=out_want, checksum=checksum,
+                outbound=ob, ntasks=ntasks, exact=int((d_ulp == 0).sum()), total=d_ulp.size)
+
+
+# ------------------------------------------------------------------- W8A8 path
+@pytest.mark.parametrize("rank", [0, 3, 7])
+def test_quant_rs_full_tiles_bit_exact(rank):
+    r = quant_case(np.random.default_rng(100 + rank), 2048, 512, 256, 8, rank)
+    assert r["exact"] == r["total"]          # same reduce order as the oracle: equality, not just 1 ulp
+
+
+def test_quant_rs_bias_fp16_out_and_full_size_peers():
+    quant_case(np.random.default_rng(1), 1024, 768, 320, 8, 5, bias=True, out_dtype=oracle.FP16, full_peers=True)
+
+
+def test_quant_rs_reference_order_int32_reduce():
+    quant_case(np.random.default_rng(2), 1024, 512, 192, 4, 1, bias=True, reduce_int32=True)
+
+
+def test_quant_rs_transposed_b():
+    quant_case(np.random.default_rng(3), 1024, 512, 256, 8, 2, trans_b=True)
+
+
+@pytest.mark.parametrize("shape", [(800, 260, 208), (8 * 130, 516, 80), (64, 256, 16), (8, 4, 16)])
+def test_quant_rs_ragged_edges(shape):
+    M, N, K = shape
+    quant_case(np.random.default_rng(4), M, N, K, 8, 6, bias=True)
+
+
+@pytest.mark.parametrize("shape", [(32, 129, 100), (24, 7, 3), (4 * 23, 45, 68), (4, 128, 512)])
+def test_quant_rs_general_shapes(shape):
+    # K not a multiple of 16 or N not a multiple of 4: the general kernel (incl. the reference's own
+    # quant test shape 4x128x512 and the 23/45/68 sizes its issue list names)
+    M, N, K = shape
+    quant_case(np.random.default_rng(5), M, N, K, 4, 3, bias=True)
+
+
+def test_quant_rs_m0_64_and_reference_launch_geometry():
+    t = ops.default_tiling(2048, 256, 1024, 8, m0=64, n0=256, k0=256, commInterval=10)
+    quant_case(np.random.default_rng(6), 2048, 1024, 256, 8, 4, tiling=t, block_num=20, stages=2)
+    t = ops.default_tiling(2048, 256, 1024, 8, m0=128, n0=256, k0=256, commInterval=2)
+    quant_case(np.random.default_rng(7), 2048, 1024, 256, 8, 4, tiling=t, block_num=4, swizzle=(3, 0), linear=True)
+
+
+def test_quant_rs_checksum_and_outbound_tiles():
+    import ctypes as C
+    M, N, K, P, rank = 2048, 512, 128, 8, 2
+    r = quant_case(np.random.default_rng(8), M, N, K, P, rank)
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    so = L.load()
+    tr, row, col, ws = (C.c_uint32() for _ in range(4))
+    cs = r["checksum"].cpu().numpy()
+    m0 = 128
+    for task in range(r["ntasks"]):
+        so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row),
+                            C.byref(col), C.byref(ws))
+        want = 0 if tr.value == rank else int(r["acc"][row.value:row.value + m0, col.value:col.value + 256].astype(np.int64).sum())
+        assert cs[task] == want, task
+    # outbound store: every non-kept tile lands at its tile-linear workspace row, dequantised in fp32
+    stages = 4  # enough stages that no round overwrites another
+    r = quant_case(np.random.default_rng(8), M, N, K, P, rank, outbound=True, stages=stages)
+    d = L.make_desc(rank, P, [16] * (P - 1), stages=stages)
+    ob = r["outbound"].cpu().numpy().reshape(-1, 256)
+    deq = oracle.dequant(r["acc"], r["s2"], r["s1"])
+    for task in range(r["ntasks"]):
+        so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row),
+                            C.byref(col), C.byref(ws))
+        if tr.value == rank:
+            continue
+        want = deq[row.value:row.value + m0, col.value:col.value + 256]
+        assert np.array_equal(ob[ws.value:ws.value + m0].view(np.uint32), want.view(np.uint32)), task
+
+
+def test_quant_fixed_config_entry_point():
+    # catcoc_quant_matmul_reduce_scatter: the example's signature (m, n, k by value, bf16 out, tile 128x256,
+    # commInterval 10); the 256-slot schedule needs 2560 % P == 0
+    import ctypes as C
+    _need_gpu()
+    rng = np.random.default_rng(9)
+    M, N, K, P, rank = 1024, 512, 128, 8, 1
+    x1 = rng.integers(-16, 16, (M, K), dtype=np.int8)       # the reference's own input range
+    x2 = rng.integers(-16, 16, (K, N), dtype=np.int8)
+    s1 = (rng.standard_normal(M) * 0.01).astype(np.float32)  # can be negative, as in gen_quant_data.py:37-38
+    s2 = (rng.standard_normal(N) * 0.01).astype(np.float32)
+    bias = np.ones(N, np.int32)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    _, want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, bias, rank * rows, rows, peers, oracle.BF16)
+    dp = [dev(p) for p in peers]
+    d = L.make_desc(rank, P, [p.data_ptr() for p in dp], peer_ld=N)
+    out = torch.zeros((rows, N), dtype=torch.bfloat16, device=DEV)
+    tx1, tx2, ts1, ts2, tb = dev(x1), dev(x2), dev(s1), dev(s2), dev(bias)
+    L.load().catcoc_quant_matmul_reduce_scatter(
+        torch.cuda.current_stream().cuda_stream, 0, tx1.data_ptr(), tx2.data_ptr(), ts1.data_ptr(), ts2.data_ptr(),
+        tb.data_ptr(), None, out.data_ptr(), C.addressof(d), M, N, K)
+    L.check()
+    torch.cuda.synchronize()
+    assert ulp_diff16(host16(out), want).max() <= 1
+
+
+def test_quant_debug_mode_closed_form_on_gpu():
+    # examples/utils/gen_quant_data.py debug data: ones, scales 0.01, bias 1..N; P identical partials
+    _need_gpu()
+    M, N, K, P = 1024, 256, 128, 8
+    rows = M // P
+    x1 = torch.ones((M, K), dtype=torch.int8, device=DEV)
+    x2 = torch.ones((K, N), dtype=torch.int8, device=DEV)
+    s1 = torch.full((M,), 0.01, dtype=torch.float32, device=DEV)
+    s2 = torch.full((N,), 0.01, dtype=torch.float32, device=DEV)
+    bias = torch.arange(1, N + 1, dtype=torch.int32, device=DEV)
+    part = ((K + bias.float()) * 0.01 * 0.01).expand(rows, N).contiguous()
+    out = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, bias, [part] * (P - 1), 0, P, out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    want = P * (K + np.arange(1, N + 1)) * 1e-4
+    assert np.allclose(out.float().cpu().numpy(), np.broadcast_to(want, (rows, N)), rtol=2 ** -9, atol=0)
+
+
+# ------------------------------------------------------------------ float paths
+def _rand16(rng, shape, dtype, scale=1.0, uniform=False):
+    x = rng.uniform(-1, 1, shape) if uniform else rng.standard_normal(shape) * scale
+    return oracle.f32_to_half(x.astype(np.float32), dtype)
+
+
+def _check_float(got_bits, want_bits, partial_f32, dtype, K):
+    got = oracle.half_to_f32(got_bits, dtype)
+    want = oracle.half_to_f32(want_bits, dtype)
+    err = np.abs(got - want) / np.maximum(1.0, np.abs(want))
+    assert err.max() <= 1e-2, "rel err %g" % err.max()      # the stated tolerance for fp32-accumulate float GEMMs
+    ok, bad, eb = oracle.verify(got, partial_f32, dtype, K)  # the reference's own gate, against unrounded fp32
+    assert ok, (bad, eb)
+
+
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+@pytest.mark.parametrize("shape", [(1024, 512, 256, 8, 3), (800, 260, 208, 8, 7), (24, 7, 30, 4, 1)])
+def test_float_reduce_scatter(dtype, shape):
+    _need_gpu()
+    M, N, K, P, rank = shape
+    rng = np.random.default_rng(20)
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    rows = M // P
+    peers = [rng.standard_normal((M, N)).astype(np.float32) for _ in range(P - 1)]   # full size, rows of the block read
+    part, want = oracle.matmul_reduce(A, B, dtype, rank * rows, rows, peers, peer_row0=rank * rows, want_partial=True)
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    out = ops.matmul_reduce_scatter(dev16(A, dtype), dev16(B, dtype), [dev(p) for p in peers], rank, P,
+                                    peer_row_offset=rank * rows, acc_dump=dump)
+    torch.cuda.synchronize()
+    full = part[rank * rows:(rank + 1) * rows] + sum(p[rank * rows:(rank + 1) * rows] for p in peers)
+    _check_float(host16(out), want, full, dtype, K)
+    pd = dump.cpu().numpy()
+    assert np.abs(pd - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
+
+
+def test_float_allreduce_config1_full_size():
+    # BASELINE config 1: A[512,2048], B[2048,1024] fp16 ~U(-1,1), K halves as the two ranks' partials
+    _need_gpu()
+    rng = np.random.default_rng(21)
+    M, N, K = 512, 1024, 2048
+    A = _rand16(rng, (M, K), oracle.FP16, uniform=True)
+    B = _rand16(rng, (K, N), oracle.FP16, uniform=True)
+    A0, B0 = np.ascontiguousarray(A[:, :K // 2]), np.ascontiguousarray(B[:K // 2])
+    p1 = oracle.gemm_half_f32(np.ascontiguousarray(A[:, K // 2:]), np.ascontiguousarray(B[K // 2:]), oracle.FP16)
+    part, want = oracle.matmul_reduce(A0, B0, oracle.FP16, 0, M, [p1], want_partial=True)
+    out = ops.matmul_allreduce(dev16(A0, oracle.FP16), dev16(B0, oracle.FP16), [dev(p1)], 0, 2)
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part + p1, oracle.FP16, K)
+    assert (ulp_diff16(host16(out), want) <= 1).mean() > 0.999
+
+
+@pytest.mark.parametrize("dtype", [oracle.BF16, oracle.FP16])
+@pytest.mark.parametrize("shape", [(256, 512, 256, 8, 2), (100, 260, 72, 4, 0), (512, 1024, 4096, 8, 5)])
+def test_allgather_matmul_reads_shards_in_place(dtype, shape):
+    _need_gpu()
+    ml, N, K, P, rank = shape
+    rng = np.random.default_rng(22)
+    shards = [_rand16(rng, (ml, K), dtype) for _ in range(P)]
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    want = oracle.allgather_matmul(shards, B, dtype)
+    dsh = [dev16(s, dtype) for s in shards]          # P separate allocations
+    out = ops.allgather_matmul(dsh[rank], [dsh[r] for r in range(P) if r != rank], dev16(B, dtype), rank, P)
+    torch.cuda.synchronize()
+    full = oracle.gemm_half_f32(np.concatenate(shards, 0), B, dtype)
+    _check_float(host16(out), want, full, dtype, K)
+
+
+def test_float_transposed_operands_general_kernel():
+    _need_gpu()
+    rng = np.random.default_rng(23)
+    M, N, K, P, rank = 256, 260, 96, 4, 2
+    A = _rand16(rng, (M, K), oracle.FP16)
+    B = _rand16(rng, (K, N), oracle.FP16, 0.05)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    part, want = oracle.matmul_reduce(A, B, oracle.FP16, rank * rows, rows, peers, want_partial=True)
+    full = part[rank * rows:(rank + 1) * rows] + sum(peers)
+    for ta, tb in ((0, 1), (1, 0), (1, 1)):
+        a = np.ascontiguousarray(A.T) if ta else A
+        b = np.ascontiguousarray(B.T) if tb else B
+        out = ops.matmul_reduce_scatter(dev16(a, oracle.FP16), dev16(b, oracle.FP16), [dev(p) for p in peers], rank, P,
+                                        trans_a=bool(ta), trans_b=bool(tb))
+        torch.cuda.synchronize()
+        _check_float(host16(out), want, full, oracle.FP16, K)
+
+
+# ------------------------------------------------------------ full benchmark size
+def test_quant_config4_full_size_properties():
+    """W8A8 benchmark config (M=8192, K=1792, N=4096, P=8) at full size.  The oracle checks a row sample
+    bit-exactly; the whole output is checked through size-independent properties: int32 accumulators
+    against torch's exact integer row/column sums, and linearity in the peer partials."""
+    _need_gpu()
+    M, N, K, P, rank = 8192, 4096, 1792, 8, 3
+    g = torch.Generator(device=DEV).manual_seed(4)
+    x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
+    x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=DEV, generator=g)
+    s1 = torch.empty(M, device=DEV).uniform_(0.005, 0.02, generator=g)
+    s2 = torch.empty(N, device=DEV).uniform_(0.001, 0.01, generator=g)
+    rows = M // P
+    peers = [torch.randn((rows, N), device=DEV, generator=g) for _ in range(P - 1)]
+    dump = torch.zeros((M, N), dtype=torch.int32, device=DEV)
+    out = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, rank, P, acc_dump=dump)
+    torch.cuda.synchronize()
+    # checksum of checksums: sum_j acc[i,j] == x1[i,:] . rowsum(x2), exact in int64
+    # (fp64 holds these integers exactly: every partial sum is below 2^53)
+    want_rows = x1.double() @ x2.double().sum(1)
+    assert torch.equal(dump.to(torch.int64).sum(1), want_rows.to(torch.int64))
+    want_cols = x1.double().sum(0) @ x2.double()
+    assert torch.equal(dump.to(torch.int64).sum(0), want_cols.to(torch.int64))
+    # oracle on a row sample of the kept block, bit for bit
+    sel = np.arange(rank * rows, (rank + 1) * rows, 37)
+    acc_s, out_s = oracle.quant_matmul_reduce_scatter(
+        x1[sel].cpu().numpy(), x2.cpu().numpy(), s1[sel].cpu().numpy(), s2.cpu().numpy(), None, 0, len(sel),
+        [p[sel - rank * rows].cpu().numpy() for p in peers], oracle.BF16)
+    assert np.array_equal(dump[sel].cpu().numpy(), acc_s)
+    assert ulp_diff16(host16(out[sel - rank * rows]), out_s).max() <= 1
+    # zero peers leave the pure dequantised block: out0 == bf16(float(acc) * s2 * s1)
+    zeros = [torch.zeros_like(peers[0])] * (P - 1)
+    out0 = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, zeros, rank, P)
+    torch.cuda.synchronize()
+    blk = dump[rank * rows:(rank + 1) * rows].float()
+    want0 = ((blk * s2[None, :]) * s1[rank * rows:(rank + 1) * rows, None]).to(torch.bfloat16)
+    assert torch.equal(out0.view(torch.int16), want0.view(torch.int16))
