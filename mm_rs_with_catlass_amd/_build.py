@@ -41,7 +41,11 @@ def build(verbose=False, extra=(), jobs=8):
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(compile_one, sources()))
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
+    # Link WITHOUT naming a HIP runtime: the library binds to the libamdhip64 its host process has
+    # already loaded (a C/C++ host links it itself; a torch process carries its own copy, and a second
+    # runtime in one process cannot open the device).
+    cxx = os.environ.get("CXX", "g++")
+    cmd = [cxx, "-shared", "-fPIC", *objs, "-o", LIB]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)

@@ -48,6 +48,9 @@ __device__ __forceinline__ typename AccOf<DT>::type mfma32(v4i a, v4i b, typenam
     }
 }
 
+__device__ __forceinline__ int f2i(float f) { return __builtin_bit_cast(int, f); }
+__device__ __forceinline__ float i2f(int i) { return __builtin_bit_cast(float, i); }
+
 // fp32 -> bf16, round to nearest even, NaN -> 0x7fc0.
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
 {
@@ -355,16 +358,22 @@ __global__ void __launch_bounds__(256, (MB <= 2) ? 2 : 1) gemm_fused_kernel(cons
                     const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
                     const float sM = (lrow < rowsK) ? args.scaleM[ti.row + lrow] : 0.f;
 #pragma unroll
-                    for (int nb = 0; nb < 4; ++nb)
-                        acc[mb][nb][r] = __builtin_bit_cast(int, __fmul_rn(__fmul_rn((float)acc[mb][nb][r], sN[nb]), sM));
+                    for (int nb = 0; nb < 4; ++nb) {
+                        const int iv = acc[mb][nb][r];
+                        acc[mb][nb][r] = f2i(__fmul_rn(__fmul_rn((float)iv, sN[nb]), sM));
+                    }
                 }
             }
         auto getf = [&](int mb, int nb, int r) -> float {
-            if constexpr (DT == DT_I8) return __builtin_bit_cast(float, acc[mb][nb][r]);
-            else return acc[mb][nb][r];
+            if constexpr (DT == DT_I8) {
+                const int iv = acc[mb][nb][r];  // bit casts go through a scalar, never a vector-element lvalue
+                return i2f(iv);
+            } else {
+                return acc[mb][nb][r];
+            }
         };
         auto setf = [&](int mb, int nb, int r, float v) {
-            if constexpr (DT == DT_I8) acc[mb][nb][r] = __builtin_bit_cast(int, v);
+            if constexpr (DT == DT_I8) acc[mb][nb][r] = f2i(v);
             else acc[mb][nb][r] = v;
         };
 

@@ -71,6 +71,27 @@ EXPORTS = [
 _lib = None
 
 
+def _preload_hip_runtime():
+    """libcatcoc_hip.so names no HIP runtime of its own; it binds to the one already in the process.
+    Make that runtime's symbols global first: torch's bundled copy when torch is importable (so that the
+    library and torch share one runtime and one set of streams), else the system ROCm one."""
+    import sys
+    cands = []
+    try:
+        import torch  # noqa: F401  (device memory and streams come from torch in this package)
+        cands.append(os.path.join(os.path.dirname(sys.modules["torch"].__file__), "lib", "libamdhip64.so"))
+    except ImportError:
+        pass
+    cands += ["/opt/rocm/lib/libamdhip64.so", "libamdhip64.so"]
+    for c in cands:
+        try:
+            C.CDLL(c, mode=C.RTLD_GLOBAL)
+            return c
+        except OSError:
+            continue
+    raise CatcocError("no HIP runtime (libamdhip64.so) could be loaded")
+
+
 def load():
     """Load libcatcoc_hip.so.  There is no fallback: a missing library is an error."""
     global _lib
@@ -80,6 +101,7 @@ def load():
         raise CatcocError(
             "libcatcoc_hip.so is not built (%s). Build it with `python -m mm_rs_with_catlass_amd._build` "
             "or __graft_entry__.build()." % LIB_PATH)
+    _preload_hip_runtime()
     L = C.CDLL(LIB_PATH)
     u32, vp = C.c_uint32, C.c_void_p
     for name in EXPORTS:
