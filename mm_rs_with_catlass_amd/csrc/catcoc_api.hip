@@ -12,6 +12,7 @@
 
 namespace catcoc {
 int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream);
+int launch_gemm_dma_i8(const GemmArgs &args, void *stream);
 int launch_gemm_f16(const GemmArgs &args, int variant, bool edge, void *stream);
 int launch_gemm_bf16(const GemmArgs &args, int variant, bool edge, void *stream);
 
@@ -60,6 +61,7 @@ struct Plan {
     bool edge;
     uint32_t dtype;
     uint32_t blockNum;
+    bool dma;     // full tiles, row-major operands: the direct-to-LDS kernel applies
 };
 
 uint32_t elem_size(uint32_t dt) { return dt == DT_I8 ? 1u : 2u; }
@@ -104,11 +106,15 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     uint32_t m0 = t->m0, n0 = t->n0;
     if (n0 == 0) n0 = 256;
     if (m0 == 0) m0 = (mRank <= 64) ? 64 : 128;
-    const bool fastShape = n0 == 256 && (m0 == 64 || m0 == 128) && !transA && t->k % che == 0 && t->n % 4 == 0;
-    plan.variant = fastShape ? (int)(m0 / 64) : 0;
+    const bool dmaShape = n0 == 256 && m0 == 256 && dt == DT_I8 && !transA && !transB && mRank % 256 == 0 && t->n % 256 == 0 &&
+                          t->k % 128 == 0 && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
+    const bool fastShape = dmaShape || n0 == 256 && (m0 == 64 || m0 == 128) && !transA && t->k % che == 0 && t->n % 4 == 0;
+    plan.variant = fastShape ? (int)(m0 / 64) : 0;   // 4 (m0 = 256) exists only as the direct-to-LDS kernel
     plan.edge = !(mRank % m0 == 0 && t->n % n0 == 0 && t->k % (64 / es) == 0);
     plan.dtype = dt;
     plan.blockNum = blockNum;
+    plan.dma = fastShape && !plan.edge && dt == DT_I8 && (m0 == 128 || m0 == 256) && !transB && !(d->flags & CATCOC_FLAG_REDUCE_INT32) &&
+               !(d->reserved0 & 16);
 
     GemmArgs &a = plan.args;
     memset(&a, 0, sizeof(a));
@@ -135,6 +141,7 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     if (op == OP_REDUCE_SCATTER) {
         a.keptBegin = d->rankIdx * mRank;
         a.keptRows = mRank;
+        a.keptRank = d->rankIdx;
         if (d->keptRows != 0 && (d->keptRowBegin != a.keptBegin || d->keptRows != a.keptRows))
             return fail(E_DESC, "explicit kept rows [%u,+%u) differ from the rank's block [%u,+%u); use the skinny-M entry for that",
                         d->keptRowBegin, d->keptRows, a.keptBegin, a.keptRows);
@@ -182,6 +189,7 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
         a.checksum = d->checksum;
     }
     a.accDump = d->accDump;
+    a.debug = d->reserved0;
     return 0;
 }
 
@@ -234,7 +242,10 @@ void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uin
     if (!check_ptr_align(p, x1, x2) || (uintptr_t)scale_x2 % 16 != 0 || (bias && (uintptr_t)bias % 16 != 0) ||
         (c_accum && (uintptr_t)c_accum % 16 != 0) || (uintptr_t)d_out % 8 != 0)
         p.variant = 0;
-    const int e = launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
+    bool dma = p.dma && p.variant != 0 && (uintptr_t)x2 % 16 == 0 && p.args.ldb % 16 == 0;
+    for (uint32_t s = 0; s < p.args.nPeers && dma; ++s) dma = (uintptr_t)p.args.peers[s] % 16 == 0;
+    if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles, 16-byte aligned row-major operands and fp32 peers"); return; }
+    const int e = dma ? launch_gemm_dma_i8(p.args, stream) : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
     ok();
 }

@@ -33,10 +33,12 @@ struct GemmArgs {
     int64_t peerLd, peerRowOffset;
     uint32_t M, N, K;              // M = rows of the local A operand
     uint32_t nPeers;
+    uint32_t keptRank;             // rank whose row block is kept (launch order puts its tiles first)
     uint32_t keptBegin, keptRows;  // global rows [keptBegin, keptBegin + keptRows) are reduced and written to d
     uint32_t flags;                // GF_*
     uint32_t outDtype;             // DT_F16 / DT_BF16
     uint32_t transA, transB;
+    uint32_t debug;                // timing experiments only (skips parts of the main loop)
     SchedParams sched;
 };
 

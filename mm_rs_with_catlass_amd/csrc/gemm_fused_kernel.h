@@ -122,7 +122,7 @@ __global__ void __launch_bounds__(256, (MB <= 2) ? 2 : 1) gemm_fused_kernel(cons
     const int c32 = lane & 31, h = lane >> 5;
 
     const SchedParams &sp = args.sched;
-    const uint32_t task = workgroup_task(blockIdx.x, sp.coreLoops, (args.flags & GF_LINEAR_ORDER) != 0);
+    const uint32_t task = launch_order_task(sp, blockIdx.x, (args.flags & GF_LINEAR_ORDER) != 0, args.keptRank);
     TileInfo ti;
     if (!task_tile(sp, task, ti)) return;
 
@@ -262,10 +262,10 @@ __global__ void __launch_bounds__(256, (MB <= 2) ? 2 : 1) gemm_fused_kernel(cons
     __syncthreads();
     for (uint32_t kt = 0; kt < nk; ++kt) {
         const bool more = kt + 1 < nk;
-        if (more) gload(kt + 1);
-        compute(kt & 1);
-        if (more) lds_store((kt + 1) & 1);
-        __syncthreads();
+        if (more && !(args.debug & 1)) gload(kt + 1);
+        if (!(args.debug & 2)) compute(kt & 1);
+        if (more && !(args.debug & 4)) lds_store((kt + 1) & 1);
+        if (!(args.debug & 8)) __syncthreads();
     }
 
     // ---- epilogue ----------------------------------------------------------

@@ -1,9 +1,23 @@
-// Instantiates the fused GEMM kernels for one element type.
+// Instantiates the fused GEMM kernels for int8 operands.
+#include "gemm_dma_kernel.h"
 #include "gemm_fused_kernel.h"
 
 namespace catcoc {
 int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream)
 {
     return launch_dt<DT_I8>(args, variant, edge, stream);
+}
+
+// Full-tile paths with direct-to-LDS copies (see gemm_dma_kernel.h for their requirements):
+// m0 = 128 (4 waves) or m0 = 256 (8 waves).
+int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
+{
+    if (args.sched.m0 == 256 && (args.debug & 32))
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, 4>), dim3(args.sched.coreLoops), dim3(512), 0, (hipStream_t)stream, args);
+    else if (args.sched.m0 == 256)
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, 2>), dim3(args.sched.coreLoops), dim3(256), 0, (hipStream_t)stream, args);
+    else
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, 2>), dim3(args.sched.coreLoops), dim3(256), 0, (hipStream_t)stream, args);
+    return (int)hipGetLastError();
 }
 }  // namespace catcoc

@@ -211,6 +211,38 @@ CATCOC_HD uint32_t workgroup_task(uint32_t wg, uint32_t tasks, bool linear)
     return ((s / CH) * X + x) * CH + s % CH;
 }
 
+// Reduce-scatter launches run the kept rank's tiles first: they are the long ones (their epilogue
+// streams the peers' partials), so starting them first lets the short tiles fill in behind them.
+// seq -> task: the kept tasks in their original order, then all others in theirs.  A bijection.
+CATCOC_HD uint32_t kept_first_task(const SchedParams &s, uint32_t keptRank, uint32_t seq)
+{
+    if (s.op != OP_REDUCE_SCATTER || s.P <= 1) return seq;
+    const uint32_t bpc = s.blockPerComm;
+    const uint32_t perRank = bpc / s.P;                 // kept tasks in a full round
+    const uint32_t fullRounds = s.coreLoops / bpc;
+    const uint32_t lastInRank = (s.coreLoops - fullRounds * bpc) / s.P;
+    const uint32_t keptCount = s.coreLoops / s.P;
+    uint32_t round, inRank, idx;
+    if (seq < keptCount) {
+        if (seq < fullRounds * perRank) { round = seq / perRank; inRank = perRank; idx = seq - round * perRank; }
+        else { round = fullRounds; inRank = lastInRank; idx = seq - fullRounds * perRank; }
+        return round * bpc + keptRank * inRank + idx;
+    }
+    const uint32_t j = seq - keptCount;
+    const uint32_t otherFull = bpc - perRank;
+    if (j < fullRounds * otherFull) { round = j / otherFull; inRank = perRank; idx = j - round * otherFull; }
+    else { round = fullRounds; inRank = lastInRank; idx = j - fullRounds * otherFull; }
+    const uint32_t b = idx < keptRank * inRank ? idx : idx + inRank;
+    return round * bpc + b;
+}
+
+// Workgroup -> task of a launch: XCD-aware chunking, then kept-first ordering.
+CATCOC_HD uint32_t launch_order_task(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank)
+{
+    if (linear) return wg;
+    return kept_first_task(s, keptRank, workgroup_task(wg, s.coreLoops, false));
+}
+
 // SplitkMatmul::GetSplitkFactor (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:219-265).
 inline uint32_t splitk_factor(uint32_t m, uint32_t n, uint32_t k, uint32_t cores, uint32_t m0, uint32_t n0,
                               uint32_t k0)

@@ -17,6 +17,7 @@ import torch
 
 from . import lib as _l
 
+_DEBUG = 0  # timing experiments only
 _TORCH_TO_DT = {torch.float16: _l.FP16, torch.bfloat16: _l.BF16}
 
 
@@ -69,6 +70,7 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
     flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_REDUCE_INT32 if reduce_int32 else 0) | \
         (_l.FLAG_LINEAR_ORDER if linear_order else 0)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
+    d.reserved0 = _DEBUG
     if out is None:
         out = torch.empty((m // max(rank_size, 1), n), dtype=out_dtype, device=x1.device)
     L = _l.load()

@@ -138,6 +138,15 @@ def test_quant_rs_m0_64_and_reference_launch_geometry():
     quant_case(np.random.default_rng(7), 2048, 1024, 256, 8, 4, tiling=t, block_num=4, swizzle=(3, 0), linear=True)
 
 
+@pytest.mark.parametrize("rank", [0, 6])
+def test_quant_rs_m0_256_eight_wave_tile(rank):
+    t = ops.default_tiling(4096, 448, 1024, 8, m0=256, n0=256, k0=256, commInterval=1)
+    r = quant_case(np.random.default_rng(30 + rank), 4096, 1024, 448, 8, rank, tiling=t, bias=True)
+    assert r["exact"] == r["total"]
+    t = ops.default_tiling(2048, 64, 512, 4, m0=256, n0=256, k0=256, commInterval=1)
+    quant_case(np.random.default_rng(32), 2048, 512, 64, 4, 1, tiling=t, outbound=True, stages=4)
+
+
 def test_quant_rs_checksum_and_outbound_tiles():
     import ctypes as C
     M, N, K, P, rank = 2048, 512, 128, 8, 2
