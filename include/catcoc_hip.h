@@ -113,7 +113,8 @@ typedef struct CatcocSymmetricDesc {
     uint32_t keptRowBegin;    /* explicit kept row range of the reduce-scatter; both 0 = rows */
     uint32_t keptRows;        /*   [rankIdx*m/rankSize, +m/rankSize) as in the reference */
     uint32_t splitK;          /* skinny-M path: k slices; 0 = GetSplitkFactor heuristic */
-    uint32_t reserved0;
+    uint32_t reduceWaitPolls; /* pre-sum path: polls (about 1 us apart) a kept tile waits for the workspace sum before it
+                                 adds the peers itself; 0 = 100000, 1 = do not wait at all */
     /* Reduce paths: peers[s], s = 0..rankSize-2, are the other ranks' partial
      * results for this rank's kept rows (fp32, or int32 with REDUCE_INT32), added
      * in slot order after the local partial.  Row `peerRowOffset + i` of a peer
@@ -127,8 +128,15 @@ typedef struct CatcocSymmetricDesc {
     uint64_t outboundBytes;   /* capacity of `outbound` */
     int64_t *checksum;        /* OUTBOUND_CHECKSUM target: one int64 per task (W8A8) / one double per task (float) */
     void *accDump;            /* optional full [m,n] int32 (W8A8) or fp32 (float) local partial, for bit-exact checks */
-    void *splitkWorkspace;    /* skinny-M path: int32 [m,n] + one uint32 per tile, zeroed by the caller once */
-    uint64_t splitkWorkspaceBytes;
+    /* Optional scratch in HBM, catcoc_get_reduce_workspace_size() bytes, 256-byte aligned, ZEROED by the caller
+     * once before its first use (the library leaves it re-armed after every launch).  With it a W8A8
+     * reduce-scatter launch on 256x256 tiles lets the workgroups of the other ranks' tiles add up the peers'
+     * partials (p0 + p1 + ... in slot order) while they compute, and the kept tiles add that one sum:
+     * d = local + (p0 + p1 + ...) instead of ((local + p0) + p1) + ..., within one output ulp of each other.
+     * Launches that share a workspace must not overlap (same stream, or ordered by events).
+     * The skinny-M path keeps its int32 split-K partials and tile counters here. */
+    void *workspace;
+    uint64_t workspaceBytes;
 } CatcocSymmetricDesc;
 
 /* ----------------------------------------------------------------------- */
@@ -198,6 +206,12 @@ CATCOC_API int catcoc_can_implement(int commType, int dataType, const CocTilingP
  * sizes layoutSymmetric = m0*commInterval*BLOCK_NUM*WORKSPACE_STAGES x n0, matmul_reduce_scatter.h:161). */
 CATCOC_API uint64_t catcoc_get_workspace_size(int commType, int dataType, const CocTilingParams *tiling,
                                               const CatcocSymmetricDesc *desc);
+
+/* Bytes of `workspace` with which this W8A8 reduce-scatter launch would pre-sum the peers' partials
+ * (fp32 [m/rankSize, n] + 256 control bytes); 0 when the shape does not qualify (it needs 256x256
+ * tiles: m/rankSize and n multiples of 256, k a multiple of 128, row-major operands, fp32 peers, at most
+ * 128 kept tiles).  No counterpart in the reference, whose reduce runs on separate vector cores. */
+CATCOC_API uint64_t catcoc_get_reduce_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc);
 
 /* Number of tasks (tiles) a launch runs; `checksum` needs this many entries. */
 CATCOC_API uint32_t catcoc_get_task_count(int commType, const CocTilingParams *tiling,

@@ -38,7 +38,14 @@ struct GemmArgs {
     uint32_t flags;                // GF_*
     uint32_t outDtype;             // DT_F16 / DT_BF16
     uint32_t transA, transB;
-    uint32_t debug;                // timing experiments only (skips parts of the main loop)
+    // Peer pre-sum of a reduce-scatter launch (NULL = off): S[keptRows, N] fp32 = sum of the peers' partials,
+    // produced by the first presumProducers workgroups of the launch sequence, consumed by the kept tiles.
+    float *presum;
+    uint32_t *presumCtl;           // [0] producers whose part of S is complete, [1] workgroups that have finished
+    uint32_t presumProducers;
+    uint32_t presumUnits;          // S in units of 8 KiB
+    uint32_t presumSpin;           // polls (about a microsecond apart) before a kept tile adds the peers itself
+    uint32_t keptTiles;
     SchedParams sched;
 };
 

@@ -2,15 +2,23 @@
 // global memory straight into LDS (no VGPR staging) three k-steps ahead of the
 // MFMAs, and the row-major B tile is transposed on the way out of LDS with the
 // transpose-read instruction, so the main loop issues almost nothing but LDS reads
-// and MFMAs.  The kept tiles' peer partials are staged through the same LDS
-// buffers, again without VGPRs, which keeps a deep queue of HBM reads in flight
-// while the accumulators stay in registers.
+// and MFMAs.
+//
+// Reduce-scatter launches have few kept tiles, and streaming the peers' partials for
+// them on a few CUs is slow (a CU sustains a small share of the HBM bandwidth).  With
+// PRESUM the NON-kept workgroups each add up a slice of the peers' partials while
+// their own main loop runs: one extra 1 KiB copy per wave per k step into a small LDS
+// ring, summed in registers and written to a scratch buffer S = p0 + p1 + ...  The
+// kept tiles run last, wait for a counter that says S is complete, and add S instead
+// of the individual peers.
 //
 // Same per-tile contract as gemm_fused_kernel (see gemm_fused_kernel.h); used when
 // every tile is full, A is [rows,K] and B is [K,N], both row-major.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "gemm_fused_kernel.h"
 
@@ -41,28 +49,40 @@ __device__ __forceinline__ void dma16(const unsigned char *g, unsigned char *lds
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(l) : "memory", "m0");
 }
 
+// 16 bytes per lane written through to device memory (device-scope store): visible to every XCD once the
+// store is acknowledged, without a write-back of the whole L2.
+__device__ __forceinline__ void store16_device(v4f v, unsigned char *g)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(g), "v"(v) : "memory");
+}
+
+// Same as dma16 with the streaming cache hint: for data that is read exactly once.
+__device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned char *lds)
+{
+    const uint32_t l = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(CATCOC_LDS unsigned char *)lds);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" : : "v"(g), "s"(l) : "memory", "m0");
+}
+
 // LDS layouts per stage (k step = 64 bytes of K):
 //   A: [row][4 x 16-byte k chunks], chunk slot = chunk ^ ((row >> 2) & 3)            (as in gemm_fused_kernel)
-//   B: raw row-major [k row][16 x 16-byte column chunks] for int8 (64 rows x 256 B),
+//   B: raw row-major [k row][16 x 16-byte column chunks] (64 rows x 256 B),
 //      column chunk slot = chunk ^ ((k row & 7) << 1); the swizzle is applied on the global side of
 //      the copy, and makes the 8-row x 16-column transpose reads of a half-wave hit all 64 banks once.
-//   fp16/bf16: 32 k rows x 512 B, 32 chunks per row, slot = chunk ^ ((k row & 3) << 1 ... see b_slot16)
 //
-// Geometries (MB = 32-row blocks per wave, WM = wave rows; every wave is 128 columns wide, two wave columns):
-//   MB 2, WM 2 -> 128x256 tile, 4 waves of 64x128, 3 stages (72 KiB LDS, two workgroups per CU);
-//   MB 2, WM 4 -> 256x256 tile, 8 waves of 64x128 (128 KiB LDS, one workgroup per CU): half the L2 -> LDS
-//                 traffic per MAC;
-//   MB 4, WM 2 -> 256x256 tile, 4 waves of 128x128, one wave per SIMD: also a third less LDS read traffic
-//                 per MFMA, which is what bounds the 64x128 waves.
-template <uint32_t DT, int MB, int WM>
-__global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(const GemmArgs args)
+// Geometries (every wave computes 64 x 128: MB = 2 row blocks of 32, 4 column blocks of 32; two wave columns):
+//   WM 2 -> 128x256 tile, 4 waves, 3 stages (72 KiB LDS, two workgroups per CU);
+//   WM 4 -> 256x256 tile, 8 waves (128 KiB LDS, one workgroup per CU): half the L2 -> LDS traffic per MAC.
+//           PRESUM (WM 4 only) adds the 32 KiB ring of the peer pre-sum.
+template <uint32_t DT, int WM, bool PRESUM>
+__global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
 {
     static_assert(DT == DT_I8, "transpose-read path is written for int8 operands");
-    static_assert((MB == 2 && (WM == 2 || WM == 4)) || (MB == 4 && WM == 2), "supported geometries");
+    static_assert(WM == 2 || WM == 4, "supported geometries");
+    static_assert(!PRESUM || WM == 4, "the pre-sum rides on the 256x256 pipeline");
     using Acc = typename AccOf<DT>::type;
+    constexpr int MB = 2;
     constexpr int NW = 2 * WM;          // waves
     constexpr int BM = 32 * MB * WM;
-    constexpr int NS = (BM == 256) ? 4 : 3;
     constexpr int A_STAGE = BM * 64;
     constexpr int B_STAGE = 64 * 256;
     constexpr int A_DMA = BM / 16 / NW;  // 1 KiB copies per wave per stage
@@ -72,13 +92,11 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
     // One LDS pool, carved by constant offsets:
     //   BM = 128: three A stages (8 KiB each), then three B stages (16 KiB each)            = 72 KiB
     //   BM = 256: two A pair buffers (32 KiB each), then four B stages (16 KiB each)         = 128 KiB
-    // After the main loop the pool is reused as per-wave staging rings for the peers' partials.
-    constexpr int NSA4 = 4, NSB4 = 4;   // BM = 256: A area = two pair buffers of 2 x 16 KiB
-    constexpr int LDS_BYTES = (BM == 256) ? (NSA4 * A_STAGE + NSB4 * B_STAGE) : 3 * (A_STAGE + B_STAGE);
+    //             PRESUM: then four ring slots of one KiB per wave                           = +32 KiB
+    constexpr int POOL = (BM == 256) ? (4 * A_STAGE + 4 * B_STAGE) : 3 * (A_STAGE + B_STAGE);
+    constexpr int RING_SLOT = NW * 1024;
+    constexpr int LDS_BYTES = POOL + (PRESUM ? 4 * RING_SLOT : 0);
     __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
-    unsigned char *const smem4 = smem;
-    unsigned char *const sA0 = smem, *const sA1 = smem + A_STAGE, *const sA2 = smem + 2 * A_STAGE;        // BM = 128
-    unsigned char *const sB0 = smem + 3 * A_STAGE, *const sB1 = sB0 + B_STAGE, *const sB2 = sB0 + 2 * B_STAGE;  // BM = 128
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -87,7 +105,10 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
     const int c32 = lane & 31, h = lane >> 5;
 
     const SchedParams &sp = args.sched;
-    const uint32_t task = launch_order_task(sp, blockIdx.x, (args.flags & GF_LINEAR_ORDER) != 0, args.keptRank);
+    const bool linear = (args.flags & GF_LINEAR_ORDER) != 0;
+    const bool presum = PRESUM && args.presum != nullptr;
+    const uint32_t seq = launch_seq(sp, blockIdx.x, linear);
+    const uint32_t task = linear ? seq : kept_order_task(sp, args.keptRank, seq, presum);
     TileInfo ti;
     if (!task_tile(sp, task, ti)) return;
 
@@ -118,10 +139,6 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
             dma16(Bgk + (size_t)row * ldbB + (((lane & 15) ^ ((row & 7) << 1)) * 16), sb + j * 1024);
         }
     };
-    auto issue = [&](unsigned char *sa, unsigned char *sb, uint32_t kt) {
-        issue_a(sa, kt);
-        issue_b(sb, kt);
-    };
 
     Acc acc[MB][4];
 #pragma unroll
@@ -132,8 +149,6 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
             for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0;
 
     // fragment addresses
-    const uint32_t a_lds = (wm * 32 * MB + c32) * 64;
-    const uint32_t a_sw = (c32 >> 2) & 3;
     // transpose read: within a 16-lane group, lane i supplies 8 bytes of k row (i>>1), column half (i&1)
     // of a 16-column chunk, and receives column i of the chunk for 8 consecutive k rows.
     const int ti16 = lane & 15, tch = (lane >> 4) & 1, trow = ti16 >> 1, thalf = ti16 & 1;
@@ -143,11 +158,6 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
         const int q = wn * 8 + nb * 2 + tch;
         b_lds[nb] = (16 * h + trow) * 256 + ((q ^ (2 * trow)) * 16) + thalf * 8;
     }
-
-    auto load_a = [&](v4i (&af)[MB], const unsigned char *sa, int kk) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) af[mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
-    };
     auto load_b = [&](v4i (&bf)[4], const unsigned char *sb, int kk) {
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
@@ -158,52 +168,133 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
         }
     };
     auto mma = [&](const v4i (&af)[MB], const v4i (&bf)[4]) {
-        if (args.debug & 2) return;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) acc[mb][nb] = mfma32<DT>(af[mb], bf[nb], acc[mb][nb]);
     };
 
+    // One k step, hand-scheduled: the 16 MFMAs of a wave are issued back to back, and every other
+    // instruction of the step (fragment reads for the NEXT eight MFMAs, the copies for later steps, the
+    // peer pre-sum) sits between two MFMAs, where it issues while the matrix pipe is busy.  The first
+    // eight MFMAs finish the previous step (fragments fa1/fb1, read during the previous step), the second
+    // eight use fa0/fb0 read during the first eight; the MFMAs lag the fragment reads by half a step, so
+    // LDS latency is never exposed.  The fences keep the compiler from regrouping the sequence.
+    v4i fa0[MB], fb0[4], fa1[MB], fb1[4];
+#define CATCOC_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define CATCOC_MMA(FA, FB, MBI, NBI)                                              \
+    acc[MBI][NBI] = mfma32<DT>(FA[MBI], FB[NBI], acc[MBI][NBI]);                  \
+    CATCOC_FENCE();
+    auto read_b1 = [&](v4i (&bf)[4], const unsigned char *sb, int kk, int nb) {
+        const unsigned char *p = sb + b_lds[nb] + kk * 32 * 256;
+        const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
+        const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 256));
+        bf[nb] = v4i{t0.x, t0.y, t1.x, t1.y};
+    };
+    // read_a(af, kk): A fragments of this step; sb: B stage of this step; slot1/2/3/4: the step's other work
+    auto sched_step = [&](auto read_a, const unsigned char *sb, auto slot1, auto slot2, auto slot3, auto slot4) {
+        CATCOC_MMA(fa1, fb1, 0, 0)
+        read_a(fa0, 0);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa1, fb1, 1, 0)
+        read_b1(fb0, sb, 0, 0);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa1, fb1, 0, 1)
+        read_b1(fb0, sb, 0, 1);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa1, fb1, 1, 1)
+        read_b1(fb0, sb, 0, 2);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa1, fb1, 0, 2)
+        read_b1(fb0, sb, 0, 3);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa1, fb1, 1, 2)
+        slot1();
+        CATCOC_FENCE();
+        CATCOC_MMA(fa1, fb1, 0, 3)
+        slot2();
+        CATCOC_FENCE();
+        CATCOC_MMA(fa1, fb1, 1, 3)
+        slot3();
+        CATCOC_FENCE();
+        CATCOC_MMA(fa0, fb0, 0, 0)
+        read_a(fa1, 1);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa0, fb0, 1, 0)
+        read_b1(fb1, sb, 1, 0);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa0, fb0, 0, 1)
+        read_b1(fb1, sb, 1, 1);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa0, fb0, 1, 1)
+        read_b1(fb1, sb, 1, 2);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa0, fb0, 0, 2)
+        read_b1(fb1, sb, 1, 3);
+        CATCOC_FENCE();
+        CATCOC_MMA(fa0, fb0, 1, 2)
+        slot4();
+        CATCOC_FENCE();
+        CATCOC_MMA(fa0, fb0, 0, 3)
+        CATCOC_MMA(fa0, fb0, 1, 3)
+    };
+#undef CATCOC_MMA
+    auto nothing = [] {};
+
     const uint32_t nk = args.K / 64;
-    if constexpr (NS == 3) {
-        // ---- 3 stages: copies run two k steps ahead; fragments are read right after the barrier ----
-        auto compute = [&](const unsigned char *sa, const unsigned char *sb) {
+    if constexpr (BM == 128) {
+        // ---- 3 stages, copies run two k steps ahead (72 KiB LDS, two workgroups per CU) ----
+        auto stA = [&](uint32_t s3) { return smem + s3 * A_STAGE; };
+        auto stB = [&](uint32_t s3) { return smem + 3 * A_STAGE + s3 * B_STAGE; };
+        const uint32_t a_lds = (wm * 32 * MB + c32) * 64;
+        const uint32_t a_sw = (c32 >> 2) & 3;
+        auto load_a = [&](v4i (&af)[MB], const unsigned char *sa, int kk) {
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-                v4i af[MB], bf[4];
-                load_a(af, sa, kk);
-                load_b(bf, sb, kk);
-                mma(af, bf);
-            }
+            for (int mb = 0; mb < MB; ++mb) af[mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
         };
-        issue(sA0, sB0, 0);
-        if (nk > 1) issue(sA1, sB1, 1);
-        uint32_t kt = 0;
-        // FULL: two more steps exist behind this one, so every condition is known to hold
-#define CATCOC_STEP(FULL, SA, SB, NA, NB)                                      \
-    {                                                                          \
-        if (FULL || kt + 1 < nk) CATCOC_WAIT_VMCNT(STEP_DMA);                  \
-        else CATCOC_WAIT_VMCNT(0);                                             \
-        barrier_keep_vmem();                                                   \
-        if (FULL || kt + 2 < nk) issue(NA, NB, kt + 2);                        \
-        compute(SA, SB);                                                       \
-        ++kt;                                                                  \
-    }
-        while (kt + 5 <= nk) {   // steps kt, kt+1, kt+2 all have two successors
-            CATCOC_STEP(1, sA0, sB0, sA2, sB2)
-            CATCOC_STEP(1, sA1, sB1, sA0, sB0)
-            CATCOC_STEP(1, sA2, sB2, sA1, sB1)
+        issue_a(stA(0), 0);
+        issue_b(stB(0), 0);
+        if (nk > 1) {
+            issue_a(stA(1), 1);
+            issue_b(stB(1), 1);
         }
-        while (true) {
-            if (kt >= nk) break;
-            CATCOC_STEP(0, sA0, sB0, sA2, sB2)
-            if (kt >= nk) break;
-            CATCOC_STEP(0, sA1, sB1, sA0, sB0)
-            if (kt >= nk) break;
-            CATCOC_STEP(0, sA2, sB2, sA1, sB1)
+        // step 0 (peeled: no MFMAs pending yet)
+        if (nk > 1) CATCOC_WAIT_VMCNT(STEP_DMA);
+        else CATCOC_WAIT_VMCNT(0);
+        barrier_keep_vmem();
+        if (nk > 2) {
+            issue_a(stA(2), 2);
+            issue_b(stB(2), 2);
         }
-#undef CATCOC_STEP
+        load_a(fa0, stA(0), 0);
+        load_b(fb0, stB(0), 0);
+        load_a(fa1, stA(0), 1);
+        load_b(fb1, stB(0), 1);
+        CATCOC_FENCE();
+        mma(fa0, fb0);
+        CATCOC_FENCE();
+        // step kt reads stage kt % 3 and refills stage (kt + 2) % 3, which every wave left at the barrier
+        uint32_t kt = 1, cur = 1, nxt = 0;
+        auto step = [&](bool more) {
+            const unsigned char *sa = stA(cur);
+            sched_step([&](v4i (&af)[MB], int kk) { load_a(af, sa, kk); }, stB(cur),
+                       [&] { if (more) issue_a(stA(nxt), kt + 2); }, [&] { if (more) issue_b(stB(nxt), kt + 2); }, nothing, nothing);
+            ++kt;
+            cur = cur == 2 ? 0 : cur + 1;
+            nxt = nxt == 2 ? 0 : nxt + 1;
+        };
+        while (kt + 2 < nk) {
+            CATCOC_WAIT_VMCNT(STEP_DMA);
+            barrier_keep_vmem();
+            step(true);
+        }
+        while (kt < nk) {
+            if (kt + 1 < nk) CATCOC_WAIT_VMCNT(STEP_DMA);
+            else CATCOC_WAIT_VMCNT(0);
+            barrier_keep_vmem();
+            step(false);
+        }
+        mma(fa1, fb1);
     } else {
         // ---- 256x256 ---------------------------------------------------------------------------------
         // B: four 64-row stages, copies issued three steps ahead.  A: two "pair" buffers of 256 rows x 128
@@ -211,15 +302,21 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
         // The MFMAs lag the fragment reads by half a step: after the barrier of step kt the fragments of
         // (kt, kk=0) are read while the MFMAs of (kt-1, kk=1) run, so LDS latency is never exposed and a
         // stage only has to have landed at its own barrier.
-        // Issue order per wave: even step [B(kt+3): 2 copies, A pair (kt+2)/2: 4 copies], odd step [B(kt+3)].
-        // At the barrier of an even step 2 copies may be in flight (B(kt+2)), at an odd step 8
-        // (B(kt+1), B(kt+2), A pair (kt+1)/2+... issued at kt-1).
+        // Copies a wave issues in step kt, in this order: B(kt+3) [B_DMA], on even kt the A pair (kt+2)/2
+        // [APC], and with PRESUM one 1 KiB piece of a peer's partial [PS].  The vector-memory counter retires
+        // in order, so "at most n outstanding" at the barrier of step s means everything older than the
+        // last n copies has landed:
+        //   even s needs A pair s/2 (issued in step s-2): younger are PS of step s-2 and all of step s-1;
+        //   odd s needs B(s) (issued in step s-3): younger are all of steps s-2 and s-1.
+        // Either way every copy of step s-3, the peer piece included, has landed at the barrier of step s.
         constexpr int AP = 256 * 128;   // bytes of an A pair buffer
-        static_assert(2 * AP == NSA4 * A_STAGE, "A pair buffers fill the A stage area");
-        auto stAP = [&](uint32_t q) { return smem4 + (q & 1) * AP; };
-        auto stB = [&](uint32_t step) { return smem4 + 2 * AP + (step & 3) * B_STAGE; };
+        constexpr int APC = 32 / NW;    // pair copies per wave
+        constexpr int PS = PRESUM ? 1 : 0;
+        constexpr int WAIT_EVEN = PS + (B_DMA + PS);
+        constexpr int WAIT_ODD = (B_DMA + PS) + (B_DMA + APC + PS);
+        auto stAP = [&](uint32_t q) { return smem + (q & 1) * AP; };
+        auto stB = [&](uint32_t step) { return smem + 2 * AP + (step & 3) * B_STAGE; };
         // pair copy j covers rows 8j..8j+7: lane -> row 8j + lane/8, slot lane&7 holds chunk slot ^ ((row>>1)&7)
-        constexpr int APC = 32 / NW;   // pair copies per wave
         auto issue_ap = [&](uint32_t q) {
             const unsigned char *Agq = Ag + (size_t)q * 128;
             unsigned char *dst = stAP(q);
@@ -237,12 +334,62 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) af[mb] = *(const v4i *)(sa + mb * 32 * 128);
         };
-        auto issue_step = [&](uint32_t kt, bool guard) {
-            if (args.debug & 1) return;
+
+        // ---- peer pre-sum state (PRESUM only) --------------------------------------------------------
+        // The scratch S is cut into units of NW KiB (one KiB per wave, within one row of S because n is a
+        // multiple of 256).  Producer i of nProd takes units i, i+nProd, ...; for each unit it copies the
+        // piece of peer 0, 1, ... in consecutive k steps, adds them in that order and stores the sum.
+        // Ring slot of the piece copied in step c is c & 3; it is added in step c + 3.
+        const uint32_t nP = args.nPeers;
+        const uint32_t nProd = args.presumProducers, nUnits = args.presumUnits;
+        const bool producer = presum && seq < nProd;
+        unsigned char *const ring = smem + POOL + w * 1024;
+        const uint32_t npr = args.N >> 8;   // KiB pieces per row of S
+        uint32_t iu = seq, ip = 0, cu = seq, cp = 0;
+        bool iact = producer && iu < nUnits, cact = iact;
+        auto unit_src = [&](uint32_t u) -> size_t {   // byte offset of this wave's piece of unit u in a peer buffer
+            const uint32_t g = u * NW + w, row = g / npr, cb = g - row * npr;
+            return ((size_t)(args.peerRowOffset + row) * args.peerLd + cb * 256) * 4 + lane * 16;
+        };
+        size_t ioff = iact ? unit_src(iu) : 0;
+        v4f psum = {0.f, 0.f, 0.f, 0.f};
+        auto peer_issue = [&](uint32_t slot) {
+            // always one copy, so the counts above hold; with nothing left to stream it re-reads cached A bytes
+            const unsigned char *src = Ag + lane * 16;
+            if (iact) {
+                src = (const unsigned char *)args.peers[ip] + ioff;
+                if (++ip == nP) {
+                    ip = 0;
+                    iu += nProd;
+                    iact = iu < nUnits;
+                    if (iact) ioff = unit_src(iu);
+                }
+            }
+            dma16_stream(src, ring + slot * RING_SLOT);
+        };
+        auto peer_read = [&](uint32_t slot) { return *(const v4f *)(ring + slot * RING_SLOT + lane * 16); };
+        auto peer_add = [&](v4f v) {
+            if (cp == 0) psum = v;
+            else {
+                psum.x = __fadd_rn(psum.x, v.x);
+                psum.y = __fadd_rn(psum.y, v.y);
+                psum.z = __fadd_rn(psum.z, v.z);
+                psum.w = __fadd_rn(psum.w, v.w);
+            }
+            if (++cp == nP) {
+                store16_device(psum, (unsigned char *)args.presum + ((size_t)cu * NW + w) * 1024 + lane * 16);
+                cp = 0;
+                cu += nProd;
+                cact = cu < nUnits;
+            }
+        };
+
+        auto issue_step_b = [&](uint32_t kt, bool guard) {
             if (!guard || kt + 3 < nk) issue_b(stB(kt + 3), kt + 3);
+        };
+        auto issue_step_a = [&](uint32_t kt, bool guard) {
             if ((kt & 1) == 0 && (!guard || kt + 2 < nk)) issue_ap((kt + 2) >> 1);
         };
-        v4i fa0[MB], fb0[4], fa1[MB], fb1[4];
         // prologue in steady-state order: B0, B1, pair 0, B2
         issue_b(stB(0), 0);
         if (nk > 1) issue_b(stB(1), 1);
@@ -252,45 +399,77 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
         if (nk > 2) CATCOC_WAIT_VMCNT(B_DMA);
         else CATCOC_WAIT_VMCNT(0);
         barrier_keep_vmem();
-        issue_step(0, true);
+        issue_step_b(0, true);
+        issue_step_a(0, true);
+        if constexpr (PRESUM) peer_issue(0);
         load_ap(fa0, 0, 0);
         load_b(fb0, stB(0), 0);
         load_ap(fa1, 0, 1);
         load_b(fb1, stB(0), 1);
-        __builtin_amdgcn_sched_barrier(0);
+        CATCOC_FENCE();
         mma(fa0, fb0);
-        __builtin_amdgcn_sched_barrier(0);
-        auto compute = [&](uint32_t kt) {
-            load_ap(fa0, kt, 0);
-            load_b(fb0, stB(kt), 0);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(fa1, fb1);      // second half of the previous step
-            __builtin_amdgcn_sched_barrier(0);
-            load_ap(fa1, kt, 1);
-            load_b(fb1, stB(kt), 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mma(fa0, fb0);
-            __builtin_amdgcn_sched_barrier(0);
+        CATCOC_FENCE();
+
+        auto compute = [&](uint32_t kt, bool guard) {
+            v4f pv;
+            bool padd = false;
+            sched_step([&](v4i (&af)[MB], int kk) { load_ap(af, kt, kk); }, stB(kt),
+                       [&] { issue_step_b(kt, guard); }, [&] { issue_step_a(kt, guard); },
+                       [&] {
+                           if constexpr (PRESUM) {
+                               peer_issue(kt & 3);
+                               padd = cact && kt >= 3;
+                               if (padd) pv = peer_read((kt - 3) & 3);
+                           }
+                       },
+                       [&] {
+                           if constexpr (PRESUM) {
+                               if (padd) peer_add(pv);
+                           }
+                       });
         };
         uint32_t kt = 1;
         for (; kt + 5 <= nk; kt += 2) {
-            CATCOC_WAIT_VMCNT(2 * B_DMA + APC);   // odd step
+            CATCOC_WAIT_VMCNT(WAIT_ODD);
             barrier_keep_vmem();
-            issue_step(kt, false);
-            compute(kt);
-            CATCOC_WAIT_VMCNT(B_DMA);           // even step
+            compute(kt, false);
+            CATCOC_WAIT_VMCNT(WAIT_EVEN);
             barrier_keep_vmem();
-            issue_step(kt + 1, false);
-            compute(kt + 1);
+            compute(kt + 1, false);
         }
         for (; kt < nk; ++kt) {   // tail: drain fully at every step
             CATCOC_WAIT_VMCNT(0);
             barrier_keep_vmem();
-            issue_step(kt, true);
-            compute(kt);
+            compute(kt, true);
         }
         mma(fa1, fb1);
+
+        if constexpr (PRESUM) {
+            if (presum) {
+                // pieces copied in the last three steps, then whatever the main loop was too short for
+                CATCOC_WAIT_VMCNT(0);
+                for (uint32_t c = nk >= 3 ? nk - 3 : 0; c < nk; ++c)
+                    if (cact) peer_add(peer_read(c & 3));
+                while (cact) {
+                    uint32_t n = 0;
+                    while (n < 4 && iact) peer_issue(n++);
+                    CATCOC_WAIT_VMCNT(0);
+                    for (uint32_t i = 0; i < n; ++i) peer_add(peer_read(i));
+                    if (n == 0) break;   // cannot happen: the two sides walk the same sequence
+                }
+                if (seq < nProd) {
+                    // make this workgroup's part of S visible to the device, then count it
+                    // S was written through to memory (device-scope stores); once they are acknowledged
+                    // the count may go up, no cache-wide write-back needed
+                    CATCOC_WAIT_VMCNT(0);
+                    __syncthreads();
+                    if (tid == 0) __hip_atomic_fetch_add(args.presumCtl, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
     }
+
+#undef CATCOC_FENCE
 
     // ---- epilogue -----------------------------------------------------------------
     // acc[mb][nb][r] is element (row, col) of the tile with
@@ -360,57 +539,61 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
                 }
             }
 
-        // peers, in slot order.  Every wave streams the peers' values for its own 64*MB/2... x 128 sub-tile
-        // through a private 16 KiB LDS ring of four 4 KiB slots, with no barriers: a sub-batch is the 8 rows of
-        // one accumulator row group (mb, r>>2) x the wave's 128 columns, copied as four 1 KiB pieces of
-        // 2 rows x 512 bytes; three sub-batches are in flight while one is added.  Pieces of rows 4..7 are
-        // stored with their 128-byte halves swapped so the two half-waves of a read hit different banks.
-        const uint32_t nP = args.nPeers;
-        if (nP != 0) {
-            static_assert(NW * 16384 <= LDS_BYTES, "peer staging rings fit the pool");
-            constexpr int SP = MB * 4;                 // sub-batches per peer; a multiple of the ring size
-            const int64_t prow0 = args.peerRowOffset + out_row0 + wm * 32 * MB;
-            unsigned char *const ring = smem + w * 16384;
-            // lane -> row (lane>>5) of the piece, 16-byte chunk (lane&31) of the wave's 512-byte row segment
-            const size_t src_lane = (size_t)(lane >> 5) * args.peerLd * 4 + (size_t)(ti.col + wn * 128) * 4;
-            auto issue_sb = [&](uint32_t p, int s) {
-                const int mb = s / 4, rq = s % 4;
-                const unsigned char *src = (const unsigned char *)args.peers[p] +
-                                           (size_t)(prow0 + mb * 32 + rq * 8) * args.peerLd * 4 + src_lane;
+        // one fp32 partial of the tile, added from global memory 32 rows (64 loads per lane) at a time
+        // (device: the partial was written by other workgroups of this launch, read it at device scope)
+        auto add_partial = [&](const float *base, int64_t ld, auto device) {
+            const float *src = base + (size_t)row_base * ld + gcol0;
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    dma16(src + (size_t)(2 * c) * args.peerLd * 4 + (((lane & 31) ^ ((c >> 1) * 8)) * 16),
-                          ring + rq * 4096 + c * 1024);
-            };
-            const uint32_t rd_lane = (2 * h) * 1024 + c32 * 4;
-            const uint32_t Q = nP * SP;
-            barrier_keep_vmem();   // every wave is done with the main loop's LDS reads
-            issue_sb(0, 0);
-            issue_sb(0, 1);
-            issue_sb(0, 2);
-            for (uint32_t p = 0; p < nP; ++p) {
+            for (int mb = 0; mb < MB; ++mb) {
+                float pv[16][4];
 #pragma unroll
-                for (int s = 0; s < SP; ++s) {
-                    const int mb = s / 4, rq = s % 4;
-                    const uint32_t ahead = Q - 1 - (p * SP + s);
-                    if (ahead >= 2) CATCOC_WAIT_VMCNT(8);
-                    else if (ahead == 1) CATCOC_WAIT_VMCNT(4);
-                    else CATCOC_WAIT_VMCNT(0);
-                    if (s + 3 < SP) issue_sb(p, s + 3);
-                    else if (p + 1 < nP) issue_sb(p + 1, s + 3 - SP);
-                    const unsigned char *slot = ring + rq * 4096 + rd_lane;
+                for (int r = 0; r < 16; ++r)
 #pragma unroll
-                    for (int ri = 0; ri < 4; ++ri) {
-                        const int r = rq * 4 + ri;
-                        const unsigned char *rowp = slot + (ri >> 1) * 1024 + (ri & 1) * 512;
-#pragma unroll
-                        for (int nb = 0; nb < 4; ++nb) {
-                            const float pv = *(const float *)(rowp + ((nb ^ h) * 128));
-                            const int iv = acc[mb][nb][r];
-                            acc[mb][nb][r] = f2i(__fadd_rn(i2f(iv), pv));
-                        }
+                    for (int nb = 0; nb < 4; ++nb) {
+                        const float *q = src + (size_t)(mb * 32 + (r >> 2) * 8 + (r & 3)) * ld + 32 * nb;
+                        if constexpr (decltype(device)::value) pv[r][nb] = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        else pv[r][nb] = __builtin_nontemporal_load(q);
                     }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb) {
+                        const int iv = acc[mb][nb][r];
+                        acc[mb][nb][r] = f2i(__fadd_rn(i2f(iv), pv[r][nb]));
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        const uint32_t nPeers = args.nPeers;
+        if (nPeers != 0) {
+            bool summed = false;
+            if constexpr (PRESUM) {
+                if (presum) {
+                    // wait (bounded) until every producer has counted its part of S
+                    volatile uint32_t *flag = (volatile uint32_t *)smem;
+                    __syncthreads();   // all waves are done with the LDS pool
+                    if (tid == 0) {
+                        uint32_t ok = 0;
+                        for (uint32_t i = 0; i < args.presumSpin; ++i) {
+                            if (__hip_atomic_load(args.presumCtl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= args.presumProducers) {
+                                ok = 1;
+                                break;
+                            }
+                            __builtin_amdgcn_s_sleep(32);
+                        }
+                        *flag = ok;
+                    }
+                    __syncthreads();
+                    summed = *flag != 0;
+
                 }
+            }
+            if (summed) {
+                add_partial(args.presum + (size_t)out_row0 * args.N, args.N, std::true_type{});
+            } else {
+                for (uint32_t p = 0; p < nPeers; ++p)
+                    add_partial((const float *)args.peers[p] + (size_t)(args.peerRowOffset + out_row0) * args.peerLd, args.peerLd, std::false_type{});
             }
         }
 
@@ -445,7 +628,7 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
                 }
             }
     } else if (args.checksum != nullptr) {
-        __shared__ long long red[NW];
+        long long *red = (long long *)smem;   // the pool is free again
         long long si = 0;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
@@ -455,6 +638,7 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
                 for (int r = 0; r < 16; ++r) si += acc[mb][nb][r];
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) si += __shfl_xor(si, o, 64);
+        __syncthreads();   // every wave has left the main loop's LDS reads behind
         if (lane == 0) red[w] = si;
         __syncthreads();
         if (tid == 0) {
@@ -462,6 +646,18 @@ __global__ void __launch_bounds__(128 * WM, (MB == 4) ? 1 : 2) gemm_dma_kernel(c
 #pragma unroll
             for (int i = 0; i < NW; ++i) t += red[i];
             ((long long *)args.checksum)[task] = t;
+        }
+    }
+
+    if constexpr (PRESUM) {
+        // the last workgroup of the launch to get here re-arms the counters for the next launch: by then
+        // every producer has counted itself and every kept tile has stopped looking at the count
+        if (presum && tid == 0) {
+            const uint32_t fin = __hip_atomic_fetch_add(args.presumCtl + 1, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+            if (fin + 1 == sp.coreLoops) {
+                __hip_atomic_store(args.presumCtl, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(args.presumCtl + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
 }

@@ -262,10 +262,10 @@ __global__ void __launch_bounds__(256, (MB <= 2) ? 2 : 1) gemm_fused_kernel(cons
     __syncthreads();
     for (uint32_t kt = 0; kt < nk; ++kt) {
         const bool more = kt + 1 < nk;
-        if (more && !(args.debug & 1)) gload(kt + 1);
-        if (!(args.debug & 2)) compute(kt & 1);
-        if (more && !(args.debug & 4)) lds_store((kt + 1) & 1);
-        if (!(args.debug & 8)) __syncthreads();
+        if (more) gload(kt + 1);
+        compute(kt & 1);
+        if (more) lds_store((kt + 1) & 1);
+        __syncthreads();
     }
 
     // ---- epilogue ----------------------------------------------------------

@@ -9,15 +9,16 @@ int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream)
 }
 
 // Full-tile paths with direct-to-LDS copies (see gemm_dma_kernel.h for their requirements):
-// m0 = 128 (4 waves) or m0 = 256 (8 waves).
+// m0 = 128 (4 waves) or m0 = 256 (8 waves, optionally with the peer pre-sum).
 int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
 {
-    if (args.sched.m0 == 256 && (args.debug & 32))
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, 4>), dim3(args.sched.coreLoops), dim3(512), 0, (hipStream_t)stream, args);
+    const dim3 grid(args.sched.coreLoops);
+    if (args.sched.m0 == 256 && args.presum != nullptr)
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, true>), grid, dim3(512), 0, (hipStream_t)stream, args);
     else if (args.sched.m0 == 256)
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, 2>), dim3(args.sched.coreLoops), dim3(256), 0, (hipStream_t)stream, args);
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, false>), grid, dim3(512), 0, (hipStream_t)stream, args);
     else
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, 2>), dim3(args.sched.coreLoops), dim3(256), 0, (hipStream_t)stream, args);
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false>), grid, dim3(256), 0, (hipStream_t)stream, args);
     return (int)hipGetLastError();
 }
 }  // namespace catcoc

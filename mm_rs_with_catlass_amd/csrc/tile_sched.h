@@ -236,6 +236,19 @@ CATCOC_HD uint32_t kept_first_task(const SchedParams &s, uint32_t keptRank, uint
     return round * bpc + b;
 }
 
+// The same with the kept tasks LAST (used when the other workgroups prepare the kept tiles' peer sum,
+// which has to be complete before a kept tile can finish).  A bijection.
+CATCOC_HD uint32_t kept_order_task(const SchedParams &s, uint32_t keptRank, uint32_t seq, bool keptLast)
+{
+    if (!keptLast || s.op != OP_REDUCE_SCATTER || s.P <= 1) return kept_first_task(s, keptRank, seq);
+    const uint32_t keptCount = s.coreLoops / s.P;
+    const uint32_t others = s.coreLoops - keptCount;
+    return kept_first_task(s, keptRank, seq < others ? seq + keptCount : seq - others);
+}
+
+// Position of a workgroup in the launch sequence (XCD-aware chunking).
+CATCOC_HD uint32_t launch_seq(const SchedParams &s, uint32_t wg, bool linear) { return workgroup_task(wg, s.coreLoops, linear); }
+
 // Workgroup -> task of a launch: XCD-aware chunking, then kept-first ordering.
 CATCOC_HD uint32_t launch_order_task(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank)
 {
