@@ -114,7 +114,8 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
                              tiles256 / P <= 128 && (t->m0 == 0 || t->m0 == 256);
     plan.presumBytes = presumShape ? (uint64_t)mRank * t->n * 4u + 256u : 0;
     const bool presum = presumShape && d->workspace != nullptr;
-    if (m0 == 0) m0 = presum ? 256 : (mRank <= 64) ? 64 : 128;
+    // measured on MI355X: 256-row tiles win once a tile has 64 or more k steps, 128-row tiles below
+    if (m0 == 0) m0 = (presum || (can256 && t->k >= 4096)) ? 256 : (mRank <= 64) ? 64 : 128;
     const bool dmaShape = can256 && m0 == 256;
     const bool fastShape = dmaShape || n0 == 256 && (m0 == 64 || m0 == 128) && !transA && t->k % che == 0 && t->n % 4 == 0;
     plan.variant = fastShape ? (int)(m0 / 64) : 0;   // 4 (m0 = 256) exists only as the direct-to-LDS kernel
