@@ -110,9 +110,10 @@ typedef struct CatcocSymmetricDesc {
     uint32_t swizzleOffset;   /* GemmIdentityBlockSwizzle<offset,direction>; 0 = <7,1> as in every example */
     uint32_t swizzleDirection;
     uint32_t flags;           /* CATCOC_OUTBOUND_* | CATCOC_FLAG_* */
-    uint32_t keptRowBegin;    /* explicit kept row range of the reduce-scatter; both 0 = rows */
-    uint32_t keptRows;        /*   [rankIdx*m/rankSize, +m/rankSize) as in the reference */
-    uint32_t splitK;          /* skinny-M path: k slices; 0 = GetSplitkFactor heuristic */
+    uint32_t keptRowBegin;    /* keptRows == 0: the rank keeps rows [rankIdx*m/rankSize, +m/rankSize) as in the reference. */
+    uint32_t keptRows;        /* keptRows != 0 (W8A8 only): the rank keeps rows [keptRowBegin, +keptRows) of an m that need not
+                                 divide by rankSize, and the launch takes the skinny-M split-K path (decode shapes) */
+    uint32_t splitK;          /* split-K path: k slices per tile; 0 = GetSplitkFactor with blockNum cores and 128x128x256 tiles */
     uint32_t reduceWaitPolls; /* pre-sum path: polls (about 1 us apart) a kept tile waits for the workspace sum before it
                                  adds the peers itself; 0 = 100000, 1 = do not wait at all */
     /* Reduce paths: peers[s], s = 0..rankSize-2, are the other ranks' partial
@@ -134,7 +135,8 @@ typedef struct CatcocSymmetricDesc {
      * partials (p0 + p1 + ... in slot order) while they compute, and the kept tiles add that one sum:
      * d = local + (p0 + p1 + ...) instead of ((local + p0) + p1) + ..., within one output ulp of each other.
      * Launches that share a workspace must not overlap (same stream, or ordered by events).
-     * The skinny-M path keeps its int32 split-K partials and tile counters here. */
+     * The split-K path keeps its int32 partial tiles and tile counters here instead
+     * (catcoc_get_splitk_workspace_size() bytes, same rules). */
     void *workspace;
     uint64_t workspaceBytes;
 } CatcocSymmetricDesc;
@@ -212,6 +214,15 @@ CATCOC_API uint64_t catcoc_get_workspace_size(int commType, int dataType, const 
  * tiles: m/rankSize and n multiples of 256, k a multiple of 128, row-major operands, fp32 peers, at most
  * 128 kept tiles).  No counterpart in the reference, whose reduce runs on separate vector cores. */
 CATCOC_API uint64_t catcoc_get_reduce_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc);
+
+/* Split-K path (descriptor with keptRows != 0): bytes of `workspace` the launch needs (0 when the split factor
+ * is 1), the split factor it will use and its number of 128x128 tiles (`checksum`, if given, needs one int64 per
+ * tile and receives the sum of the accumulators of the tile's rows that are not kept).  The path takes row-major
+ * int8 A [m,k] and B [k,n], k % 64 == 0, n % 128 == 0, fp32 peers [keptRows, n].  It stands in for
+ * SplitkMatmul (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:68-330) in front of the
+ * dequant / reduce epilogue. */
+CATCOC_API uint64_t catcoc_get_splitk_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
+                                                     uint32_t *splitK, uint32_t *tiles);
 
 /* Number of tasks (tiles) a launch runs; `checksum` needs this many entries. */
 CATCOC_API uint32_t catcoc_get_task_count(int commType, const CocTilingParams *tiling,

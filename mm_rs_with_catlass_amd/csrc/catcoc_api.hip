@@ -13,6 +13,7 @@
 namespace catcoc {
 int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream);
 int launch_gemm_dma_i8(const GemmArgs &args, void *stream);
+int launch_gemm_splitk_i8(const GemmArgs &args, int rowBlocks, uint32_t tasks, void *stream);
 int launch_gemm_f16(const GemmArgs &args, int variant, bool edge, void *stream);
 int launch_gemm_bf16(const GemmArgs &args, int variant, bool edge, void *stream);
 
@@ -150,9 +151,6 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
         a.keptBegin = d->rankIdx * mRank;
         a.keptRows = mRank;
         a.keptRank = d->rankIdx;
-        if (d->keptRows != 0 && (d->keptRowBegin != a.keptBegin || d->keptRows != a.keptRows))
-            return fail(E_DESC, "explicit kept rows [%u,+%u) differ from the rank's block [%u,+%u); use the skinny-M entry for that",
-                        d->keptRowBegin, d->keptRows, a.keptBegin, a.keptRows);
     } else if (op == OP_ALLREDUCE) {
         a.keptBegin = 0;
         a.keptRows = t->m;
@@ -242,12 +240,113 @@ void launch_float(int commType, int dataType, void *stream, uint8_t *a, uint8_t 
     ok();
 }
 
+// ---- skinny-M split-K path (explicit kept rows) ----------------------------------------------
+struct SplitkPlan {
+    GemmArgs args;
+    uint32_t f, tiles, rowBlocks;
+    uint64_t workspaceBytes;   // partial tiles + counters (0 when f == 1)
+};
+
+int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uint32_t transA, uint32_t transB, SplitkPlan &sp)
+{
+    if (t == nullptr) return fail(E_NULL, "tiling is NULL");
+    if (d == nullptr || d->magic != CATCOC_DESC_MAGIC) return fail(E_DESC, "symmetricPtr does not point at a CatcocSymmetricDesc");
+    if (t->m == 0 || t->n == 0 || t->k == 0) return fail(E_SHAPE, "empty problem m=%u n=%u k=%u", t->m, t->n, t->k);
+    const uint32_t P = d->rankSize;
+    if (P == 0 || P > CATCOC_MAX_RANKS) return fail(E_RANK, "rankSize %u out of range 1..%d", P, CATCOC_MAX_RANKS);
+    if (transA || transB) return fail(E_SHAPE, "the explicit-kept-rows (split-K) path takes row-major A [m,k] and B [k,n] only");
+    if (t->k % 64 != 0 || t->n % 128 != 0)
+        return fail(E_SHAPE, "the explicit-kept-rows (split-K) path needs k %% 64 == 0 and n %% 128 == 0 (k=%u, n=%u)", t->k, t->n);
+    if ((t->m0 != 0 && t->m0 != 128) || (t->n0 != 0 && t->n0 != 128))
+        return fail(E_TILING, "the split-K path runs 128x128 tiles; leave m0/n0 zero or pass 128 (m0=%u, n0=%u)", t->m0, t->n0);
+    if (d->keptRows == 0 || (uint64_t)d->keptRowBegin + d->keptRows > t->m)
+        return fail(E_DESC, "kept rows [%u,+%u) outside [0,%u)", d->keptRowBegin, d->keptRows, t->m);
+    if (d->flags & CATCOC_FLAG_REDUCE_INT32) return fail(E_DESC, "the split-K path reduces fp32 peers after the dequant only");
+    if ((d->flags & CATCOC_OUTBOUND_MASK) == CATCOC_OUTBOUND_STORE)
+        return fail(E_DESC, "the split-K path folds non-kept rows into checksums; CATCOC_OUTBOUND_STORE is not supported there");
+    const uint32_t off = d->swizzleOffset ? d->swizzleOffset : 7u;
+    const uint32_t dir = d->swizzleOffset ? d->swizzleDirection : 1u;
+    if (dir > 1) return fail(E_TILING, "swizzleDirection %u must be 0 or 1", dir);
+
+    GemmArgs &a = sp.args;
+    memset(&a, 0, sizeof(a));
+    a.M = t->m; a.N = t->n; a.K = t->k;
+    a.lda = t->k; a.ldb = t->n; a.ldd = t->n;
+    a.outDtype = DT_BF16;
+    a.sched.off = off; a.sched.dir = dir;
+    a.keptBegin = d->keptRowBegin;
+    a.keptRows = d->keptRows;
+    a.nPeers = P - 1;
+    for (uint32_t s = 0; s < a.nPeers; ++s) {
+        if (d->peers[s] == nullptr) return fail(E_NULL, "reduce needs %u staged peer partials; peers[%u] is NULL", a.nPeers, s);
+        a.peers[s] = d->peers[s];
+    }
+    a.peerLd = d->peerLd ? d->peerLd : t->n;
+    a.peerRowOffset = d->peerRowOffset;
+    if (a.nPeers && a.peerLd < (int64_t)t->n) return fail(E_DESC, "peerLd %lld < n %u", (long long)a.peerLd, t->n);
+    if (a.peerRowOffset < 0) return fail(E_DESC, "peerRowOffset must be >= 0");
+    a.checksum = d->checksum;
+    a.accDump = d->accDump;
+
+    const uint32_t cores = d->blockNum ? d->blockNum : kDefaultBlockNum;
+    const uint32_t kTiles = ceil_div(t->k, 256u);
+    sp.tiles = ceil_div(t->m, 128u) * (t->n / 128u);
+    uint32_t f = d->splitK ? d->splitK : splitk_factor(t->m, t->n, t->k, cores, 128, 128, 256);
+    if (f > kTiles) f = kTiles;
+    if (f == 0) f = 1;
+    sp.f = f;
+    a.splitK = f;
+    sp.rowBlocks = t->m <= 32 ? 1 : t->m <= 64 ? 2 : 4;
+    sp.workspaceBytes = f > 1 ? (uint64_t)f * sp.tiles * 128u * 128u * 4u + (uint64_t)((sp.tiles * 4u + 255u) / 256u) * 256u : 0;
+    return 0;
+}
+
+void launch_quant_splitk(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias,
+                         uint8_t *c_accum, uint8_t *d_out, const CatcocSymmetricDesc *d, CocTilingParams *tiling,
+                         uint32_t transA, uint32_t transB, uint32_t outDataType)
+{
+    SplitkPlan sp;
+    if (make_splitk_plan(tiling, d, transA, transB, sp)) return;
+    if (!x1 || !x2 || !scale_x1 || !scale_x2 || !d_out) { fail(E_NULL, "x1, x2, scale_x1, scale_x2 and d_out must be non-NULL"); return; }
+    if (outDataType != FP16 && outDataType != BF16) { fail(E_DTYPE, "outDataType %u must be FP16 (1) or BF16 (27)", outDataType); return; }
+    if ((uintptr_t)x1 % 16 != 0 || (uintptr_t)x2 % 16 != 0 || sp.args.lda % 16 != 0 || sp.args.ldb % 16 != 0) {
+        fail(E_SHAPE, "the split-K path needs 16-byte aligned x1, x2 and row pitches");
+        return;
+    }
+    GemmArgs &a = sp.args;
+    if (sp.f > 1) {
+        if (d->workspace == nullptr || d->workspaceBytes < sp.workspaceBytes) {
+            fail(E_WORKSPACE, "split factor %u needs a zero-initialised workspace of %llu bytes (catcoc_get_splitk_workspace_size)",
+                 sp.f, (unsigned long long)sp.workspaceBytes);
+            return;
+        }
+        if ((uintptr_t)d->workspace % 256 != 0) { fail(E_WORKSPACE, "workspace must be 256-byte aligned"); return; }
+        a.skPart = (int32_t *)d->workspace;
+        a.skCount = (uint32_t *)((unsigned char *)d->workspace + (uint64_t)sp.f * sp.tiles * 128u * 128u * 4u);
+    }
+    a.a[0] = x1;
+    a.b = x2;
+    a.d = d_out;
+    a.scaleM = (const float *)scale_x1;
+    a.scaleN = (const float *)scale_x2;
+    a.bias = (const int32_t *)bias;
+    a.cAccum = (int32_t *)c_accum;
+    a.outDtype = outDataType;
+    const int e = launch_gemm_splitk_i8(a, (int)sp.rowBlocks, sp.tiles * sp.f, stream);
+    if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
+    ok();
+}
+
 void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias,
                   uint8_t *c_accum, uint8_t *d_out, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA,
                   uint32_t transB, uint32_t outDataType)
 {
     Plan p;
     const CatcocSymmetricDesc *d = (const CatcocSymmetricDesc *)symmetricPtr;
+    if (d != nullptr && d->magic == CATCOC_DESC_MAGIC && d->keptRows != 0) {
+        launch_quant_splitk(stream, x1, x2, scale_x1, scale_x2, bias, c_accum, d_out, d, tiling, transA, transB, outDataType);
+        return;
+    }
     if (make_plan(QUANT_MATMUL_REDUCE_SCATTER, INT8, tiling, d, transA, transB, p)) return;
     if (!x1 || !x2 || !scale_x1 || !scale_x2 || !d_out) { fail(E_NULL, "x1, x2, scale_x1, scale_x2 and d_out must be non-NULL"); return; }
     if (outDataType != FP16 && outDataType != BF16) { fail(E_DTYPE, "outDataType %u must be FP16 (1) or BF16 (27)", outDataType); return; }
@@ -366,6 +465,21 @@ uint64_t catcoc_get_reduce_workspace_size(const CocTilingParams *tiling, const C
     if (make_plan(QUANT_MATMUL_REDUCE_SCATTER, INT8, tiling, &d, 0, 0, p)) return 0;
     ok();
     return p.presumBytes;
+}
+
+uint64_t catcoc_get_splitk_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t *splitK,
+                                          uint32_t *tiles)
+{
+    SplitkPlan sp;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
+    d = *desc;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    if (make_splitk_plan(tiling, &d, 0, 0, sp)) return 0;
+    ok();
+    if (splitK) *splitK = sp.f;
+    if (tiles) *tiles = sp.tiles;
+    return sp.workspaceBytes;
 }
 
 uint32_t catcoc_get_task_count(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc)

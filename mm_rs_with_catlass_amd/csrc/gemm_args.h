@@ -46,6 +46,10 @@ struct GemmArgs {
     uint32_t presumUnits;          // S in units of 8 KiB
     uint32_t presumSpin;           // polls (about a microsecond apart) before a kept tile adds the peers itself
     uint32_t keptTiles;
+    // Skinny-M split-K launch: k slices per tile, int32 partial tiles [splitK][tiles][128][128], one counter per tile.
+    uint32_t splitK;
+    int32_t *skPart;
+    uint32_t *skCount;
     SchedParams sched;
 };
 

@@ -1,0 +1,14 @@
+// Instantiates the skinny-M split-K W8A8 kernel.
+#include "gemm_splitk_kernel.h"
+
+namespace catcoc {
+// rowBlocks: 32-row blocks of A a tile stages (1, 2 or 4); grid = tiles x k slices.
+int launch_gemm_splitk_i8(const GemmArgs &args, int rowBlocks, uint32_t tasks, void *stream)
+{
+    const dim3 grid(tasks), block(256);
+    if (rowBlocks == 1) hipLaunchKernelGGL((gemm_splitk_kernel<1>), grid, block, 0, (hipStream_t)stream, args);
+    else if (rowBlocks == 2) hipLaunchKernelGGL((gemm_splitk_kernel<2>), grid, block, 0, (hipStream_t)stream, args);
+    else hipLaunchKernelGGL((gemm_splitk_kernel<4>), grid, block, 0, (hipStream_t)stream, args);
+    return (int)hipGetLastError();
+}
+}  // namespace catcoc

@@ -61,7 +61,7 @@ EXPORTS = [
     "catcoc_launch_matmul_reduce_scatter_fp16", "catcoc_launch_matmul_reduce_scatter_bf16",
     "catcoc_quant_matmul_reduce_scatter", "catcoc_launch_quant_matmul_reduce_scatter",
     "catcoc_last_error", "catcoc_last_status", "catcoc_can_implement", "catcoc_get_workspace_size",
-    "catcoc_get_reduce_workspace_size",
+    "catcoc_get_reduce_workspace_size", "catcoc_get_splitk_workspace_size",
     "catcoc_get_task_count", "catcoc_get_tilings", "catcoc_check_comm_interval_reduce_scatter",
     "catcoc_check_comm_interval_allreduce", "catcoc_check_comm_interval_allgather", "catcoc_get_splitk_factor",
     "catcoc_default_tiling", "catcoc_swizzle_block_coord", "catcoc_splitk_block_coord", "catcoc_splitk_actual_k",
@@ -105,6 +105,7 @@ def load():
     _preload_hip_runtime()
     L = C.CDLL(LIB_PATH)
     u32, vp = C.c_uint32, C.c_void_p
+    pu = C.POINTER(u32)
     for name in EXPORTS:
         if name.startswith("catcoc_launch_") and name != "catcoc_launch_quant_matmul_reduce_scatter":
             f = getattr(L, name)
@@ -125,6 +126,8 @@ def load():
     L.catcoc_get_workspace_size.restype = C.c_uint64
     L.catcoc_get_reduce_workspace_size.argtypes = [C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc)]
     L.catcoc_get_reduce_workspace_size.restype = C.c_uint64
+    L.catcoc_get_splitk_workspace_size.argtypes = [C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), pu, pu]
+    L.catcoc_get_splitk_workspace_size.restype = C.c_uint64
     L.catcoc_get_task_count.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc)]
     L.catcoc_get_task_count.restype = u32
     L.catcoc_get_tilings.argtypes = [C.POINTER(CocTilingParams), C.c_int, C.c_int, C.c_int, C.POINTER(CocTilingParams), C.c_int]
@@ -138,7 +141,6 @@ def load():
     L.catcoc_get_splitk_factor.restype = u32
     L.catcoc_default_tiling.argtypes = [C.POINTER(CocTilingParams), u32, u32, u32, u32]
     L.catcoc_default_tiling.restype = None
-    pu = C.POINTER(u32)
     L.catcoc_swizzle_block_coord.argtypes = [u32] * 5 + [pu, pu]
     L.catcoc_splitk_block_coord.argtypes = [u32] * 7 + [pu] * 4
     L.catcoc_splitk_actual_k.argtypes = [u32] * 4

@@ -110,6 +110,54 @@ def quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
     return out
 
 
+def splitk_plan(m, k, n, rank_size, kept_row_begin, kept_rows, split_k=0, block_num=0):
+    """(workspace bytes, split factor, 128x128 tiles) of the skinny-M split-K path for this problem."""
+    t = default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
+    d = _l.make_desc(0, rank_size, block_num=block_num)
+    d.keptRowBegin, d.keptRows, d.splitK = kept_row_begin, kept_rows, split_k
+    f, tiles = C.c_uint32(), C.c_uint32()
+    need = _l.load().catcoc_get_splitk_workspace_size(C.byref(t), C.byref(d), C.byref(f), C.byref(tiles))
+    _l.check()
+    return int(need), f.value, tiles.value
+
+
+def prepare_quant_matmul_splitk(x1, x2, scale_x1, scale_x2, bias=None, peers=(), rank_size=1, kept_row_begin=0,
+                                kept_rows=None, out_dtype=torch.bfloat16, split_k=0, workspace=None, checksum=None,
+                                acc_dump=None, c_accum=None, peer_row_offset=0, block_num=0, swizzle=None, out=None):
+    """Skinny-M (decode) form of the W8A8 operator: x1 [m,k] with any m, the rank keeps rows
+    [kept_row_begin, +kept_rows); peers are rank_size-1 fp32 partials [kept_rows, n].  Returns (launch, out)."""
+    _check_dev(x1, x2, scale_x1, scale_x2, bias, checksum, acc_dump, c_accum, workspace, *peers)
+    m, k = x1.shape
+    n = x2.shape[1]
+    t = default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
+    d = _desc(0, rank_size, list(peers), peer_row_offset, 0, block_num, 0, swizzle, None, checksum, acc_dump)
+    d.keptRowBegin = kept_row_begin
+    d.keptRows = kept_rows if kept_rows is not None else m
+    d.splitK = split_k
+    if workspace is not None:
+        d.workspace = workspace.data_ptr()
+        d.workspaceBytes = workspace.numel() * workspace.element_size()
+    if out is None:
+        out = torch.empty((d.keptRows, n), dtype=out_dtype, device=x1.device)
+    keep = (x1, x2, scale_x1, scale_x2, bias, tuple(peers), checksum, acc_dump, c_accum, out, d, t, workspace)
+    fn = _l.load().catcoc_launch_quant_matmul_reduce_scatter
+    argv = (0, x1.data_ptr(), x2.data_ptr(), scale_x1.data_ptr(), scale_x2.data_ptr(), _ptr(bias), _ptr(c_accum),
+            out.data_ptr(), C.addressof(d), C.byref(t), 0, 0, _TORCH_TO_DT[out.dtype])
+
+    def launch(_keep=keep):
+        fn(_stream(), *argv)
+
+    return launch, out
+
+
+def quant_matmul_splitk(*args, **kw):
+    """One launch of prepare_quant_matmul_splitk(); returns d_out [kept_rows, n]."""
+    launch, out = prepare_quant_matmul_splitk(*args, **kw)
+    launch()
+    _l.check()
+    return out
+
+
 def reduce_workspace_size(m, k, n, rank, rank_size, tiling=None):
     """Bytes of the optional pre-sum workspace of quant_matmul_reduce_scatter (0 = this shape cannot use one)."""
     t = tiling if tiling is not None else default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)

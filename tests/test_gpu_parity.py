@@ -198,6 +198,63 @@ def test_quant_rs_presum_wait_gives_up_and_adds_peers_itself():
     assert r["exact"] == r["total"]
 
 
+@pytest.mark.parametrize("case", [(1, 512, 1024, 8, 0, 1, 0), (16, 512, 2048, 8, 0, 2, 0), (16, 384, 1024, 8, 6, 10, 4),
+                                  (64, 256, 4096, 8, 8, 8, 0), (128, 640, 2048, 8, 112, 16, 0), (200, 256, 1088, 4, 100, 50, 3),
+                                  (33, 128, 64, 2, 0, 33, 0), (512, 1024, 1024, 8, 0, 64, 2)])
+def test_quant_skinny_m_splitk(case):
+    # decode shapes: any m, explicit kept rows, k slices meet through the workspace; int32 sums are exact
+    _need_gpu()
+    M, N, K, P, kb, kr, f = case
+    rng = np.random.default_rng(60 + M)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.integers(-1000, 1000, N, dtype=np.int32)
+    peers = [rng.standard_normal((kr, N)).astype(np.float32) for _ in range(P - 1)]
+    acc_want, out_want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, b, kb, kr, peers, oracle.BF16)
+    need, fac, tiles = ops.splitk_plan(M, K, N, P, kb, kr, split_k=f)
+    assert tiles == -(-M // 128) * (N // 128) and fac >= 1 and (f == 0 or fac == min(f, -(-K // 256)))
+    ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=DEV)
+    acc_dump = torch.full((M, N), -7, dtype=torch.int32, device=DEV)
+    c_accum = torch.full((kr, N), -7, dtype=torch.int32, device=DEV)
+    checksum = torch.zeros(tiles, dtype=torch.int64, device=DEV)
+    launch, out = ops.prepare_quant_matmul_splitk(dev(x1), dev(x2), dev(s1), dev(s2), dev(b), [dev(p) for p in peers], P,
+                                                  kb, kr, split_k=f, workspace=ws, checksum=checksum, acc_dump=acc_dump,
+                                                  c_accum=c_accum)
+    for it in range(2):                      # the second launch reuses the workspace the first one re-armed
+        out.zero_()
+        launch()
+        L.check()
+        torch.cuda.synchronize()
+        assert np.array_equal(acc_dump.cpu().numpy(), acc_want), "int32 accumulators differ from the oracle"
+        assert np.array_equal(c_accum.cpu().numpy(), acc_want[kb:kb + kr])
+        assert np.array_equal(host16(out), out_want), "kept rows differ from the oracle"
+    cs = checksum.cpu().numpy()
+    keep = np.zeros(M, bool)
+    keep[kb:kb + kr] = True
+    for t in range(tiles):
+        mi, ni = divmod(t, N // 128)
+        blk = acc_want[mi * 128:(mi + 1) * 128, ni * 128:(ni + 1) * 128].astype(np.int64)
+        assert cs[t] == blk[~keep[mi * 128:(mi + 1) * 128]].sum(), t
+
+
+def test_quant_skinny_m_rejections():
+    _need_gpu()
+    x1 = torch.zeros((16, 96), dtype=torch.int8, device=DEV)
+    x2 = torch.zeros((96, 256), dtype=torch.int8, device=DEV)
+    s1 = torch.ones(16, device=DEV)
+    s2 = torch.ones(256, device=DEV)
+    with pytest.raises(L.CatcocError, match="k % 64"):
+        ops.quant_matmul_splitk(x1, x2, s1, s2, None, [], 1, 0, 2)
+    x1 = torch.zeros((16, 2048), dtype=torch.int8, device=DEV)
+    x2 = torch.zeros((2048, 256), dtype=torch.int8, device=DEV)
+    with pytest.raises(L.CatcocError, match="workspace"):
+        ops.quant_matmul_splitk(x1, x2, s1, s2, None, [], 1, 0, 2, split_k=4)
+    with pytest.raises(L.CatcocError, match="kept rows"):
+        ops.quant_matmul_splitk(x1, x2, s1, s2, None, [], 1, 10, 7, split_k=1)
+
+
 def test_quant_rs_checksum_and_outbound_tiles():
     import ctypes as C
     M, N, K, P, rank = 2048, 512, 128, 8, 2
