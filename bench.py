@@ -8,6 +8,7 @@ in HBM before the timed region.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode kept|outbound] [--no-cpu]
     python bench.py --mode copy     # plain 256 MiB device copy: the known-size kernel the HBM counters are scaled by
+    python bench.py --mode decode   # BASELINE config 5: skinny-M sweep, K = N = 8192, GB/s per M (HBM-bound)
 """
 import argparse
 import json
@@ -48,12 +49,69 @@ def cpu_baseline(M, N, K, P, rank, repeats):
                                                                                     sum(ts) / len(ts))}
 
 
+def decode_sweep(args, torch, L, ops, dev):
+    """BASELINE config 5: A [M,8192] int8, B [8192,8192] int8 (64 MiB, the dominant traffic), P = 8, rank 0 keeps
+    rows [0, ceil(M/8)).  B rotates over six copies (384 MiB) so the 256 MB Infinity Cache cannot serve it."""
+    import numpy as np
+    import oracle
+    K = N = 8192
+    P, copies = 8, 6
+    g = torch.Generator(device=dev).manual_seed(20250101)
+    Bs = [torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g) for _ in range(copies)]
+    s2 = torch.empty(N, device=dev).uniform_(0.001, 0.01, generator=g)
+    sweep = []
+    for M in (1, 16, 64, 128, 512):
+        kr = -(-M // P)
+        x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
+        s1 = torch.empty(M, device=dev).uniform_(0.005, 0.02, generator=g)
+        peers = [torch.randn((kr, N), device=dev, generator=g) for _ in range(P - 1)]
+        need, f, tiles = ops.splitk_plan(M, K, N, P, 0, kr)
+        ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=dev)
+        out = torch.empty((kr, N), dtype=torch.bfloat16, device=dev)
+        steps = [ops.prepare_quant_matmul_splitk(x1, b, s1, s2, None, peers, P, 0, kr, workspace=ws, out=out)[0] for b in Bs]
+        steps[0]()
+        L.check()
+        for i in range(args.warmup):
+            steps[i % copies]()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(args.steps):
+            steps[i % copies]()
+        e1.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / args.steps
+        kern = e0.elapsed_time(e1) / args.steps / 1e3
+        # parity of the last launch (B copy (steps-1) % copies) against the oracle
+        bl = Bs[(args.steps - 1) % copies]
+        _, want = oracle.quant_matmul_reduce_scatter(x1[:kr].cpu().numpy(), bl.cpu().numpy(), s1[:kr].cpu().numpy(), s2.cpu().numpy(),
+                                                     None, 0, kr, [p.cpu().numpy() for p in peers], oracle.BF16, want_acc=False)
+        ok = bool(np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), want))
+        alg = K * N + M * K + 4 * (M + N) + (P - 1) * kr * N * 4 + kr * N * 2
+        sweep.append({"M": M, "kept_rows": kr, "split_k": f, "tiles": tiles, "kernel_us": round(kern * 1e6, 2),
+                      "wall_us": round(wall * 1e6, 2), "algorithmic_bytes": alg, "GBps": round(alg / kern / 1e9, 1),
+                      "hbm_frac": round(alg / kern / 1e9 / PEAK_HBM_GBS, 4), "TOPS": round(2.0 * M * N * K / kern / 1e12, 2),
+                      "parity_ok": ok})
+    hbm = [r for r in sweep if r["M"] <= 128]
+    worst = min(hbm, key=lambda r: r["GBps"])
+    print(json.dumps({
+        "metric": "W8A8 decode sweep (BASELINE config 5) algorithmic GB/s per M, 1 MI355X", "value": worst["GBps"],
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": worst["wall_us"] / 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "W8A8 skinny-M matmul + reduce epilogue, K=N=8192, P=8, M in {1,16,64,128,512}; value = lowest GB/s over M <= 128",
+                   "b_copies_rotated": copies},
+        "roofline": {"bound": "hbm", "achieved": worst["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(worst["GBps"] / PEAK_HBM_GBS, 4), "traffic": None},
+        "sweep": sweep}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--mode", choices=["kept", "outbound", "copy"], default="kept",
+    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode"], default="kept",
                     help="kept: non-kept tiles are folded into checksums (BASELINE's literal outputs); "
                          "outbound: they are also stored as fp32 to the symmetric workspace")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -89,6 +147,9 @@ def main():
         dt = (time.perf_counter() - t0) / args.steps
         print(json.dumps({"metric": "device copy", "bytes_read": nbytes, "bytes_written": nbytes, "steps": args.steps,
                           "ms_per_step": round(dt * 1e3, 5), "value": round(2 * nbytes / dt / 1e9, 1), "unit": "GB/s"}))
+        return
+    if args.mode == "decode":
+        decode_sweep(args, torch, L, ops, dev)
         return
     M, K, N, P, rank = 8192, 1792, 4096, 8, args.rank
     rows = M // P

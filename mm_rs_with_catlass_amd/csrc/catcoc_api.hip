@@ -285,6 +285,8 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
     a.peerRowOffset = d->peerRowOffset;
     if (a.nPeers && a.peerLd < (int64_t)t->n) return fail(E_DESC, "peerLd %lld < n %u", (long long)a.peerLd, t->n);
     if (a.peerRowOffset < 0) return fail(E_DESC, "peerRowOffset must be >= 0");
+    if ((uint64_t)(a.peerRowOffset + a.keptRows) * (uint64_t)a.peerLd * 4u > 0x7fffffffull)
+        return fail(E_DESC, "the split-K path addresses each peer partial with 31-bit byte offsets: (peerRowOffset + keptRows) * peerLd * 4 must stay below 2 GiB");
     a.checksum = d->checksum;
     a.accDump = d->accDump;
 

@@ -60,8 +60,14 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     const unsigned char *Bg = (const unsigned char *)args.b + (size_t)kBeg * ldb + colT;
 
     // A: copy j covers tile rows 16j..16j+15; lane -> row 16j + lane/4, LDS chunk slot lane&3 holds k chunk slot^swz
-    auto issue = [&](uint32_t st, uint32_t kt) {
+    // Every workgroup of a k slice reads the same 64-byte column of A at the same step, and the rows of A are a
+    // power of two apart, so those reads would all queue at one L2 channel.  Each workgroup therefore walks its k
+    // steps from a different starting point (integer sums do not care about the order); workgroups that share an
+    // XCD (blockIdx mod 8) get consecutive starting points, which spreads them over the channels.
+    const uint32_t rot = (blockIdx.x >> 3) % nsteps;
+    auto issue = [&](uint32_t st, uint32_t step) {
         unsigned char *sa = smem + st * STAGE, *sb = sa + A_STAGE;
+        const uint32_t kt = step + rot < nsteps ? step + rot : step + rot - nsteps;
         const unsigned char *Agk = Ag + (size_t)kt * 64;
         const unsigned char *Bgk = Bg + (size_t)kt * 64 * ldb;
 #pragma unroll
@@ -109,34 +115,46 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         // stage (kt + NS - 1) % NS was read in step kt - 1, which every wave has left
         if (kt + NS - 1 < nsteps) issue((kt + NS - 1) & (NS - 1), kt + NS - 1);
         const unsigned char *sa = smem + (kt & (NS - 1)) * STAGE, *sb = sa + A_STAGE;
+        // all fragment reads of the step first, then the MFMAs: one LDS round trip per step instead of one per
+        // 32-row block (left to itself the compiler reuses two fragment registers and serialises them)
+        v4i bf[2], af[2][MBW];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
             const unsigned char *p = sb + b_lds + kk * 32 * 128;
             const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
             const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 128));
-            const v4i bf = v4i{t0.x, t0.y, t1.x, t1.y};
+            bf[kk] = v4i{t0.x, t0.y, t1.x, t1.y};
 #pragma unroll
-            for (int mb = 0; mb < MBW; ++mb) {
-                const v4i af = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
-                acc[mb] = mfma32<DT_I8>(af, bf, acc[mb]);
-            }
+            for (int mb = 0; mb < MBW; ++mb)
+                af[kk][mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int mb = 0; mb < MBW; ++mb) acc[mb] = mfma32<DT_I8>(af[kk][mb], bf[kk], acc[mb]);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- k slices meet -------------------------------------------------------------
     // acc[mb][r] is element (lrow, lcol) with lrow = mb*32 + (r>>2)*8 + h*4 + (r&3), lcol = w*32 + c32
     const uint32_t lcol = w * 32 + c32;
     if (f > 1) {
-        int32_t *part = args.skPart + ((size_t)slice * loopsM * loopsN + tile) * (128 * 128) + lcol;
+        // Partial tiles travel through memory at device scope (cache policy sc1: written through / read past
+        // the XCD-local L2), as ordinary buffer accesses so that the loads of a slice are issued together.
+        constexpr int DEVICE_SCOPE = 16;   // sc1
+        const size_t tileBytes = 128 * 128 * 4;
+        const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(args.skPart + ((size_t)slice * loopsM * loopsN + tile) * (128 * 128)), 0, (int)tileBytes, 0x00020000);
 #pragma unroll
         for (int mb = 0; mb < MBW; ++mb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const uint32_t lrow = mb * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
                 const int iv = acc[mb][r];
-                if (lrow < rowsValid) __hip_atomic_store(part + lrow * 128, iv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (lrow < rowsValid) __builtin_amdgcn_raw_buffer_store_b32(iv, mine, (lrow * 128 + lcol) * 4, 0, DEVICE_SCOPE);
             }
-        // the partial is written through to memory; once the stores are acknowledged the slice may be counted
+        // once the stores are acknowledged the slice may be counted
         CATCOC_WAIT_VMCNT(0);
         __syncthreads();
         volatile uint32_t *flag = (volatile uint32_t *)smem;
@@ -144,44 +162,90 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         __syncthreads();
         if (*flag != f - 1u) return;
         if (tid == 0) __hip_atomic_store(args.skCount + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for (uint32_t s = 0; s < f; ++s) {
-            if (s == slice) continue;
-            const int32_t *other = args.skPart + ((size_t)s * loopsM * loopsN + tile) * (128 * 128) + lcol;
+        // the other slices' partials, one 32-row block at a time and up to four slices per round trip
+        const int32_t *tile0 = args.skPart + (size_t)tile * (128 * 128);
+        const size_t sliceStride = (size_t)loopsM * loopsN * (128 * 128);
 #pragma unroll
-            for (int mb = 0; mb < MBW; ++mb)
+        for (int mb = 0; mb < MBW; ++mb) {
+            for (uint32_t s0 = 0; s0 < f; s0 += 4) {
+                int pv[4][16];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const uint32_t lrow = mb * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
-                    if (lrow < rowsValid) acc[mb][r] += __hip_atomic_load(other + lrow * 128, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t s = s0 + q;
+                    const bool use = s < f && s != slice;
+                    const __amdgpu_buffer_rsrc_t other = __builtin_amdgcn_make_buffer_rsrc(
+                        (void *)(tile0 + (use ? s : slice) * sliceStride), 0, (int)tileBytes, 0x00020000);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t lrow = mb * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
+                        // unused slots and rows past the end read as zero: the offset is pushed out of the descriptor's range
+                        pv[q][r] = __builtin_amdgcn_raw_buffer_load_b32(other, (use && lrow < rowsValid) ? (lrow * 128 + lcol) * 4 : 0x7fffffff, 0, DEVICE_SCOPE);
+                    }
                 }
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[mb][r] += pv[q][r];
+            }
         }
     }
 
     // ---- epilogue on the rows that exist -----------------------------------------------
+    // Per 32-row block: bias, dumps, dequant; then the peers' values of the block's kept rows are fetched eight
+    // peers at a time in ONE round trip (out-of-range offsets of a buffer load cost nothing and return zero, which
+    // masks rows that are not kept and peers that do not exist) and added in slot order; then the 16-bit store.
     const uint32_t gcol = colT + lcol;
     const int bv = args.bias ? args.bias[gcol] : 0;
     const float sN = args.scaleN[gcol];
+    const uint32_t keptEnd = args.keptBegin + args.keptRows;
+    const uint64_t peerBytes = (uint64_t)(args.peerRowOffset + args.keptRows) * args.peerLd * 4;
+    const int peerRange = peerBytes > 0x7fffffffull ? 0x7fffffff : (int)peerBytes;
     long long csum = 0;
 #pragma unroll
-    for (int mb = 0; mb < MBW; ++mb)
+    for (int mb = 0; mb < MBW; ++mb) {
+        const uint32_t blk0 = row0 + mb * 32;
+        if (blk0 >= row0 + rowsValid) break;
+        float v[16];
+        uint32_t poff[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const uint32_t lrow = mb * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
-            if (lrow >= rowsValid) continue;
             const uint32_t grow = row0 + lrow;
+            const bool valid = lrow < rowsValid;
+            const bool kept = valid && grow >= args.keptBegin && grow < keptEnd;
             const int iv = acc[mb][r] + bv;
-            if (args.accDump) ((int32_t *)args.accDump)[(size_t)grow * N + gcol] = iv;
-            if (grow >= args.keptBegin && grow < args.keptBegin + args.keptRows) {
-                const uint32_t orow = grow - args.keptBegin;
-                if (args.cAccum) args.cAccum[(size_t)orow * N + gcol] = iv;
-                float v = __fmul_rn(__fmul_rn((float)iv, sN), args.scaleM[grow]);
-                for (uint32_t p = 0; p < args.nPeers; ++p)
-                    v = __fadd_rn(v, __builtin_nontemporal_load((const float *)args.peers[p] + (size_t)(args.peerRowOffset + orow) * args.peerLd + gcol));
-                ((unsigned short *)args.d)[(size_t)orow * args.ldd + gcol] = (unsigned short)f32_to_out16(v, args.outDtype);
-            } else {
-                csum += iv;
+            if (valid && args.accDump) ((int32_t *)args.accDump)[(size_t)grow * N + gcol] = iv;
+            if (kept && args.cAccum) args.cAccum[(size_t)(grow - args.keptBegin) * N + gcol] = iv;
+            if (valid && !kept) csum += iv;
+            v[r] = __fmul_rn(__fmul_rn((float)iv, sN), args.scaleM[valid ? grow : row0]);
+            poff[r] = kept ? (uint32_t)(((args.peerRowOffset + grow - args.keptBegin) * args.peerLd + gcol) * 4) : 0x7fffffffu;
+        }
+        if (blk0 < keptEnd && blk0 + 32 > args.keptBegin) {   // the block holds kept rows
+            for (uint32_t p0 = 0; p0 < args.nPeers; p0 += 8) {
+                float pv[8][16];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const bool use = p0 + q < args.nPeers;
+                    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+                        (void *)args.peers[use ? p0 + q : 0], 0, use ? peerRange : 0, 0x00020000);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        pv[q][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, poff[r], 0, 2 /* streaming */));
+                }
+#pragma unroll
+                for (int q = 0; q < 8; ++q)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (p0 + q < args.nPeers) v[r] = __fadd_rn(v[r], pv[q][r]);
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t grow = blk0 + (r >> 2) * 8 + h * 4 + (r & 3);
+                if (poff[r] != 0x7fffffffu)
+                    ((unsigned short *)args.d)[(size_t)(grow - args.keptBegin) * args.ldd + gcol] = (unsigned short)f32_to_out16(v[r], args.outDtype);
             }
         }
+    }
     if (args.checksum != nullptr) {
         long long *red = (long long *)smem + 8;
 #pragma unroll
