@@ -56,6 +56,12 @@ __device__ __forceinline__ void store16_device(v4f v, unsigned char *g)
     asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(g), "v"(v) : "memory");
 }
 
+// The same with the LDS destination given as a byte address that is already wave-uniform (built from scalars).
+__device__ __forceinline__ void dma16_at(const unsigned char *g, uint32_t ldsAddr)
+{
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(ldsAddr) : "memory", "m0");
+}
+
 // Same as dma16 with the streaming cache hint: for data that is read exactly once.
 __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned char *lds)
 {
@@ -119,24 +125,35 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const unsigned char *Bg = (const unsigned char *)args.b + ti.col;
 
     // ---- copy descriptors ---------------------------------------------------
-    // A: copy j covers rows 16j..16j+15; lane -> row 16j + lane/4, LDS chunk slot lane&3 holds k chunk slot^swz
-    const uint32_t a_goff = (uint32_t)(lane >> 2) * (uint32_t)ldaB + (((lane & 3) ^ ((lane >> 4) & 3)) * 16);
-    // B: copy j covers k rows 4j..4j+3; lane -> row 4j + lane/16, LDS slot lane&15 holds column chunk slot^((row&7)<<1)
-    auto issue_a = [&](unsigned char *sa, uint32_t kt) {
-        const unsigned char *Agk = Ag + (size_t)kt * 64;
+    // Every copy a wave issues has its own global pointer, advanced after each issue, and a scalar LDS address:
+    // issuing a copy is then a pointer add, an M0 write and the load.  Steps are issued in increasing order.
+    const uint32_t ws = __builtin_amdgcn_readfirstlane((uint32_t)w);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(CATCOC_LDS unsigned char *)smem;
+    // A (128-row tiles): copy j covers rows 16j..16j+15; lane -> row 16j + lane/4, LDS chunk slot lane&3 holds k chunk slot^swz
+    const unsigned char *gA[A_DMA];
+#pragma unroll
+    for (int jj = 0; jj < A_DMA; ++jj)
+        gA[jj] = Ag + (size_t)(16 * (w + NW * jj) + (lane >> 2)) * ldaB + (((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+    auto issue_a = [&](uint32_t ldsStage) {   // next k step of A into the stage at LDS byte offset ldsStage
 #pragma unroll
         for (int jj = 0; jj < A_DMA; ++jj) {
-            const int j = w + NW * jj;
-            dma16(Agk + (size_t)(16 * j) * ldaB + a_goff, sa + j * 1024);
+            dma16_at(gA[jj], lds0 + ldsStage + (ws + NW * jj) * 1024);
+            gA[jj] += 64;
         }
     };
-    auto issue_b = [&](unsigned char *sb, uint32_t kt) {
-        const unsigned char *Bgk = Bg + (size_t)kt * 64 * ldbB;
+    // B: copy j covers k rows 4j..4j+3; lane -> row 4j + lane/16, LDS slot lane&15 holds column chunk slot^((row&7)<<1)
+    const unsigned char *gB[B_DMA];
+#pragma unroll
+    for (int jj = 0; jj < B_DMA; ++jj) {
+        const int row = 4 * (w + NW * jj) + (lane >> 4);
+        gB[jj] = Bg + (size_t)row * ldbB + (((lane & 15) ^ ((row & 7) << 1)) * 16);
+    }
+    const size_t bStep = (size_t)64 * ldbB;
+    auto issue_b = [&](uint32_t ldsStage) {   // next k step of B
 #pragma unroll
         for (int jj = 0; jj < B_DMA; ++jj) {
-            const int j = w + NW * jj;
-            const int row = 4 * j + (lane >> 4);
-            dma16(Bgk + (size_t)row * ldbB + (((lane & 15) ^ ((row & 7) << 1)) * 16), sb + j * 1024);
+            dma16_at(gB[jj], lds0 + ldsStage + (ws + NW * jj) * 1024);
+            gB[jj] += bStep;
         }
     };
 
@@ -246,25 +263,27 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         // ---- 3 stages, copies run two k steps ahead (72 KiB LDS, two workgroups per CU) ----
         auto stA = [&](uint32_t s3) { return smem + s3 * A_STAGE; };
         auto stB = [&](uint32_t s3) { return smem + 3 * A_STAGE + s3 * B_STAGE; };
+        auto offA = [&](uint32_t s3) { return s3 * A_STAGE; };
+        auto offB = [&](uint32_t s3) { return 3 * A_STAGE + s3 * B_STAGE; };
         const uint32_t a_lds = (wm * 32 * MB + c32) * 64;
         const uint32_t a_sw = (c32 >> 2) & 3;
         auto load_a = [&](v4i (&af)[MB], const unsigned char *sa, int kk) {
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) af[mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
         };
-        issue_a(stA(0), 0);
-        issue_b(stB(0), 0);
+        issue_a(offA(0));
+        issue_b(offB(0));
         if (nk > 1) {
-            issue_a(stA(1), 1);
-            issue_b(stB(1), 1);
+            issue_a(offA(1));
+            issue_b(offB(1));
         }
         // step 0 (peeled: no MFMAs pending yet)
         if (nk > 1) CATCOC_WAIT_VMCNT(STEP_DMA);
         else CATCOC_WAIT_VMCNT(0);
         barrier_keep_vmem();
         if (nk > 2) {
-            issue_a(stA(2), 2);
-            issue_b(stB(2), 2);
+            issue_a(offA(2));
+            issue_b(offB(2));
         }
         load_a(fa0, stA(0), 0);
         load_b(fb0, stB(0), 0);
@@ -278,7 +297,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         auto step = [&](bool more) {
             const unsigned char *sa = stA(cur);
             sched_step([&](v4i (&af)[MB], int kk) { load_a(af, sa, kk); }, stB(cur),
-                       [&] { if (more) issue_a(stA(nxt), kt + 2); }, [&] { if (more) issue_b(stB(nxt), kt + 2); }, nothing, nothing);
+                       [&] { if (more) issue_a(offA(nxt)); }, [&] { if (more) issue_b(offB(nxt)); }, nothing, nothing);
             ++kt;
             cur = cur == 2 ? 0 : cur + 1;
             nxt = nxt == 2 ? 0 : nxt + 1;
@@ -317,16 +336,20 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         auto stAP = [&](uint32_t q) { return smem + (q & 1) * AP; };
         auto stB = [&](uint32_t step) { return smem + 2 * AP + (step & 3) * B_STAGE; };
         // pair copy j covers rows 8j..8j+7: lane -> row 8j + lane/8, slot lane&7 holds chunk slot ^ ((row>>1)&7)
-        auto issue_ap = [&](uint32_t q) {
-            const unsigned char *Agq = Ag + (size_t)q * 128;
-            unsigned char *dst = stAP(q);
+        const unsigned char *gP[APC];
+#pragma unroll
+        for (int jj = 0; jj < APC; ++jj) {
+            const int row = 8 * (w + NW * jj) + (lane >> 3);
+            gP[jj] = Ag + (size_t)row * ldaB + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+        }
+        auto issue_ap = [&](uint32_t q) {   // pairs are issued in increasing q
 #pragma unroll
             for (int jj = 0; jj < APC; ++jj) {
-                const int j = w + NW * jj;
-                const int row = 8 * j + (lane >> 3);
-                dma16(Agq + (size_t)row * ldaB + (((lane & 7) ^ ((row >> 1) & 7)) * 16), dst + j * 1024);
+                dma16_at(gP[jj], lds0 + (q & 1) * AP + (ws + NW * jj) * 1024);
+                gP[jj] += 128;
             }
         };
+        auto offB4 = [&](uint32_t step) { return 2 * AP + (step & 3) * B_STAGE; };
         const uint32_t ap_lds = (wm * 32 * MB + c32) * 128;
         const uint32_t ap_sw = (c32 >> 1) & 7;
         auto load_ap = [&](v4i (&af)[MB], uint32_t kt, int kk) {
@@ -385,16 +408,16 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         };
 
         auto issue_step_b = [&](uint32_t kt, bool guard) {
-            if (!guard || kt + 3 < nk) issue_b(stB(kt + 3), kt + 3);
+            if (!guard || kt + 3 < nk) issue_b(offB4(kt + 3));
         };
         auto issue_step_a = [&](uint32_t kt, bool guard) {
             if ((kt & 1) == 0 && (!guard || kt + 2 < nk)) issue_ap((kt + 2) >> 1);
         };
         // prologue in steady-state order: B0, B1, pair 0, B2
-        issue_b(stB(0), 0);
-        if (nk > 1) issue_b(stB(1), 1);
+        issue_b(offB4(0));
+        if (nk > 1) issue_b(offB4(1));
         issue_ap(0);
-        if (nk > 2) issue_b(stB(2), 2);
+        if (nk > 2) issue_b(offB4(2));
         // step 0 (peeled: no MFMAs pending yet)
         if (nk > 2) CATCOC_WAIT_VMCNT(B_DMA);
         else CATCOC_WAIT_VMCNT(0);
@@ -413,8 +436,12 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         auto compute = [&](uint32_t kt, bool guard) {
             v4f pv;
             bool padd = false;
+            // The two waves that share a SIMD (w and w + 4) issue their copies in different halves of the step,
+            // so that one of them always has MFMAs to feed the matrix pipe while the other computes addresses.
+            // (With the pre-sum every wave keeps the order B, A pair, peer piece that the wait counts assume.)
+            const bool early = PRESUM || ws < NW / 2;
             sched_step([&](v4i (&af)[MB], int kk) { load_ap(af, kt, kk); }, stB(kt),
-                       [&] { issue_step_b(kt, guard); }, [&] { issue_step_a(kt, guard); },
+                       [&] { if (early) issue_step_b(kt, guard); }, [&] { if (early) issue_step_a(kt, guard); },
                        [&] {
                            if constexpr (PRESUM) {
                                peer_issue(kt & 3);
@@ -425,6 +452,11 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
                        [&] {
                            if constexpr (PRESUM) {
                                if (padd) peer_add(pv);
+                           } else {
+                               if (!early) {
+                                   issue_step_b(kt, guard);
+                                   issue_step_a(kt, guard);
+                               }
                            }
                        });
         };
