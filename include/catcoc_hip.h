@@ -274,6 +274,12 @@ CATCOC_API void catcoc_comm_block_idx(uint32_t dir, uint32_t P, uint32_t splitRo
 CATCOC_API int catcoc_task_tile(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
                                 uint32_t task, uint32_t *targetRank, uint32_t *row, uint32_t *col,
                                 uint32_t *wsRow);
+/* The task workgroup `wg` of a launch runs: XCD-aware chunking, then the kept rank's tiles first (they are the
+ * long ones), or last when the descriptor carries a pre-sum workspace.  A bijection on [0, task count);
+ * 0xffffffff for wg out of range or rejected arguments.  No counterpart in the reference, where AI core i
+ * simply runs tasks i, i + BLOCK_NUM, ... (quant_matmul_reduce_scatter.hpp:166-170). */
+CATCOC_API uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
+                                       uint32_t wg);
 /* The task workgroup `wg` of a launch with `tasks` tasks runs (XCD-aware chunking unless
  * CATCOC_FLAG_LINEAR_ORDER); a bijection on [0,tasks). */
 CATCOC_API uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags);

@@ -519,6 +519,24 @@ int catcoc_task_tile(int commType, const CocTilingParams *tiling, const CatcocSy
     return 1;
 }
 
+uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t wg)
+{
+    Plan p;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0xffffffffu; }
+    d = *desc;
+    d.flags &= ~CATCOC_OUTBOUND_MASK;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    const int dataType = commType == QUANT_MATMUL_REDUCE_SCATTER ? INT8 : FP16;
+    if (make_plan(commType, dataType, tiling, &d, 0, 0, p)) return 0xffffffffu;
+    ok();
+    const SchedParams &s = p.args.sched;
+    if (wg >= s.coreLoops) return 0xffffffffu;
+    const bool linear = (p.args.flags & GF_LINEAR_ORDER) != 0;
+    const uint32_t seq = launch_seq(s, wg, linear);
+    return linear ? seq : kept_order_task(s, p.args.keptRank, seq, p.args.presum != nullptr);
+}
+
 uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags)
 {
     return workgroup_task(wg, tasks, (flags & CATCOC_FLAG_LINEAR_ORDER) != 0);

@@ -65,7 +65,7 @@ EXPORTS = [
     "catcoc_get_task_count", "catcoc_get_tilings", "catcoc_check_comm_interval_reduce_scatter",
     "catcoc_check_comm_interval_allreduce", "catcoc_check_comm_interval_allgather", "catcoc_get_splitk_factor",
     "catcoc_default_tiling", "catcoc_swizzle_block_coord", "catcoc_splitk_block_coord", "catcoc_splitk_actual_k",
-    "catcoc_allgather_block_coord", "catcoc_comm_block_idx", "catcoc_task_tile", "catcoc_workgroup_task",
+    "catcoc_allgather_block_coord", "catcoc_comm_block_idx", "catcoc_task_tile", "catcoc_workgroup_task", "catcoc_launch_task",
     "catcoc_device_info", "catcoc_version",
 ]
 
@@ -128,6 +128,8 @@ def load():
     L.catcoc_get_reduce_workspace_size.restype = C.c_uint64
     L.catcoc_get_splitk_workspace_size.argtypes = [C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), pu, pu]
     L.catcoc_get_splitk_workspace_size.restype = C.c_uint64
+    L.catcoc_launch_task.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32]
+    L.catcoc_launch_task.restype = u32
     L.catcoc_get_task_count.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc)]
     L.catcoc_get_task_count.restype = u32
     L.catcoc_get_tilings.argtypes = [C.POINTER(CocTilingParams), C.c_int, C.c_int, C.c_int, C.POINTER(CocTilingParams), C.c_int]

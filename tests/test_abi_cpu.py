@@ -124,6 +124,47 @@ def test_workgroup_task_is_a_bijection(so):
         assert per == [16] * 8
 
 
+def test_launch_order_is_a_bijection_with_kept_tiles_first_or_last(so):
+    from mm_rs_with_catlass_amd import ops
+    for (M, K, N, P, rank, m0) in [(8192, 1792, 4096, 8, 0, 128), (8192, 1792, 4096, 8, 5, 256), (2048, 256, 1024, 4, 3, 128)]:
+        t = ops.default_tiling(M, K, N, P, m0=m0, n0=256, k0=256)
+        for ws in (False, True):
+            d = L.make_desc(rank, P)
+            if ws:
+                d.workspace, d.workspaceBytes = 4096, 1 << 40    # never dereferenced on the host
+            n = so.catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+            tasks = [so.catcoc_launch_task(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), wg) for wg in range(n)]
+            assert sorted(tasks) == list(range(n))
+            assert so.catcoc_launch_task(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), n) == 0xffffffff
+            tr = u32()
+            kept = []
+            for task in tasks:
+                so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), None, None, None)
+                kept.append(tr.value == rank)
+            nk = sum(kept)
+            assert nk == n // P
+            presum = ws and m0 == 256          # the pre-sum rides on 256-row tiles only
+            # XCD chunking permutes positions inside blocks of 128 workgroups, so compare block-wise
+            pos = sorted(so.catcoc_workgroup_task(wg, n, 0) for wg in range(n) if kept[wg])
+            assert pos == (list(range(n - nk, n)) if presum else list(range(nk)))
+
+
+def test_workspace_size_queries(so):
+    from mm_rs_with_catlass_amd import ops
+    assert ops.reduce_workspace_size(8192, 1792, 4096, 0, 8) == 1024 * 4096 * 4 + 256
+    assert ops.reduce_workspace_size(8192, 1792 + 64, 4096, 0, 8) == 0          # k not a multiple of 128
+    assert ops.reduce_workspace_size(8192 + 8, 1792, 4096, 0, 8) == 0           # ragged rows
+    need, f, tiles = ops.splitk_plan(16, 8192, 8192, 8, 0, 2)
+    assert (f, tiles) == (oracle.splitk_factor(16, 8192, 8192, 256, 128, 128, 256), 64)
+    assert need == f * tiles * 128 * 128 * 4 + 256
+    need, f, tiles = ops.splitk_plan(512, 8192, 8192, 8, 0, 64)
+    assert (need, f, tiles) == (0, 1, 256)
+    need, f, tiles = ops.splitk_plan(200, 1088, 256, 4, 100, 50, split_k=3)
+    assert (f, tiles) == (3, 4) and need == 3 * 4 * 65536 + 256
+    with pytest.raises(L.CatcocError, match="kept rows"):
+        ops.splitk_plan(16, 8192, 8192, 8, 10, 7)
+
+
 def test_tiling_search_equals_oracle(so):
     for ct, octx in ((L.MATMUL_ALLREDUCE, oracle.MATMUL_ALLREDUCE), (L.ALLGATHER_MATMUL, oracle.ALLGATHER_MATMUL),
                      (L.MATMUL_REDUCE_SCATTER, oracle.MATMUL_REDUCE_SCATTER)):
