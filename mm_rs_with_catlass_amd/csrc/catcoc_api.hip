@@ -16,6 +16,8 @@ int launch_gemm_dma_i8(const GemmArgs &args, void *stream);
 int launch_gemm_splitk_i8(const GemmArgs &args, int rowBlocks, uint32_t tasks, void *stream);
 int launch_gemm_f16(const GemmArgs &args, int variant, bool edge, void *stream);
 int launch_gemm_bf16(const GemmArgs &args, int variant, bool edge, void *stream);
+int launch_gemm_dma_f16(const GemmArgs &args, void *stream);
+int launch_gemm_dma_bf16(const GemmArgs &args, void *stream);
 
 static int launch_gemm(uint32_t dtype, const GemmArgs &args, int variant, bool edge, void *stream)
 {
@@ -107,23 +109,23 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     // tile selection: the fast kernels have n0 = 256 and m0 in {64,128}, or 256 for W8A8 on full tiles
     uint32_t m0 = t->m0, n0 = t->n0;
     if (n0 == 0) n0 = 256;
-    const bool can256 = n0 == 256 && dt == DT_I8 && !transA && !transB && mRank % 256 == 0 && t->n % 256 == 0 &&
-                        t->k % 128 == 0 && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
+    const bool can256 = n0 == 256 && !transA && !transB && mRank % 256 == 0 && t->n % 256 == 0 &&
+                        ((uint64_t)t->k * es) % 128 == 0 && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
     // the peer pre-sum needs 256-row tiles, few enough kept tiles to be resident together, and other tiles to do it
     const uint32_t tiles256 = can256 ? (t->m / 256) * (t->n / 256) : 0;
-    const bool presumShape = can256 && op == OP_REDUCE_SCATTER && P > 1 && !(d->flags & CATCOC_FLAG_LINEAR_ORDER) &&
+    const bool presumShape = can256 && dt == DT_I8 && op == OP_REDUCE_SCATTER && P > 1 && !(d->flags & CATCOC_FLAG_LINEAR_ORDER) &&
                              tiles256 / P <= 128 && (t->m0 == 0 || t->m0 == 256);
     plan.presumBytes = presumShape ? (uint64_t)mRank * t->n * 4u + 256u : 0;
     const bool presum = presumShape && d->workspace != nullptr;
-    // measured on MI355X: 256-row tiles win once a tile has 64 or more k steps, 128-row tiles below
-    if (m0 == 0) m0 = (presum || (can256 && t->k >= 4096)) ? 256 : (mRank <= 64) ? 64 : 128;
+    // measured on MI355X: two 128x256 workgroups per CU beat one 256x256 workgroup at every k tried
+    if (m0 == 0) m0 = presum ? 256 : (mRank <= 64) ? 64 : 128;
     const bool dmaShape = can256 && m0 == 256;
     const bool fastShape = dmaShape || n0 == 256 && (m0 == 64 || m0 == 128) && !transA && t->k % che == 0 && t->n % 4 == 0;
     plan.variant = fastShape ? (int)(m0 / 64) : 0;   // 4 (m0 = 256) exists only as the direct-to-LDS kernel
     plan.edge = !(mRank % m0 == 0 && t->n % n0 == 0 && t->k % (64 / es) == 0);
     plan.dtype = dt;
     plan.blockNum = blockNum;
-    plan.dma = fastShape && !plan.edge && dt == DT_I8 && (m0 == 128 || m0 == 256) && !transB && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
+    plan.dma = fastShape && !plan.edge && (m0 == 128 || m0 == 256) && !transA && !transB && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
 
     GemmArgs &a = plan.args;
     memset(&a, 0, sizeof(a));
@@ -235,7 +237,10 @@ void launch_float(int commType, int dataType, void *stream, uint8_t *a, uint8_t 
     p.args.b = b;
     p.args.d = c;
     if (!check_ptr_align(p, a, b)) p.variant = 0;
-    const int e = launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
+    const bool dma = p.dma && p.variant != 0 && (uintptr_t)b % 16 == 0 && (p.args.ldb * 2) % 16 == 0;
+    if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles and 16-byte aligned row-major operands"); return; }
+    const int e = dma ? (p.dtype == DT_F16 ? launch_gemm_dma_f16(p.args, stream) : launch_gemm_dma_bf16(p.args, stream))
+                      : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
     ok();
 }

@@ -24,6 +24,8 @@
 
 namespace catcoc {
 
+typedef short v4s16 __attribute__((ext_vector_type(4)));
+
 #define CATCOC_LDS __attribute__((address_space(3)))
 #define CATCOC_GLB __attribute__((address_space(1)))
 
@@ -82,10 +84,10 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 template <uint32_t DT, int WM, bool PRESUM>
 __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
 {
-    static_assert(DT == DT_I8, "transpose-read path is written for int8 operands");
     static_assert(WM == 2 || WM == 4, "supported geometries");
-    static_assert(!PRESUM || WM == 4, "the pre-sum rides on the 256x256 pipeline");
+    static_assert(!PRESUM || (WM == 4 && DT == DT_I8), "the pre-sum rides on the 256x256 W8A8 pipeline");
     using Acc = typename AccOf<DT>::type;
+    constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
     constexpr int MB = 2;
     constexpr int NW = 2 * WM;          // waves
     constexpr int BM = 32 * MB * WM;
@@ -118,11 +120,11 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     TileInfo ti;
     if (!task_tile(sp, task, ti)) return;
 
-    const int64_t ldaB = args.lda, ldbB = args.ldb;  // int8: elements == bytes
+    const int64_t ldaB = args.lda * ES, ldbB = args.ldb * ES;  // row pitches in bytes
     const bool gather = sp.op == OP_ALLGATHER;
     const unsigned char *Ag = (const unsigned char *)args.a[gather ? ti.targetRank : 0] +
                               (int64_t)(gather ? ti.rowInRank : ti.row) * ldaB;
-    const unsigned char *Bg = (const unsigned char *)args.b + ti.col;
+    const unsigned char *Bg = (const unsigned char *)args.b + (size_t)ti.col * ES;
 
     // ---- copy descriptors ---------------------------------------------------
     // Every copy a wave issues has its own global pointer, advanced after each issue, and a scalar LDS address:
@@ -141,14 +143,21 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             gA[jj] += 64;
         }
     };
-    // B: copy j covers k rows 4j..4j+3; lane -> row 4j + lane/16, LDS slot lane&15 holds column chunk slot^((row&7)<<1)
+    // B, 1-byte elements: copy j covers k rows 4j..4j+3; lane -> row 4j + lane/16, LDS slot lane&15 holds column
+    // chunk slot^((row&7)<<1).  2-byte elements (32 k rows x 512 bytes): copy j covers k rows 2j, 2j+1; lane -> row
+    // 2j + lane/32, slot lane&31 holds chunk slot^((row&3)<<2).
     const unsigned char *gB[B_DMA];
 #pragma unroll
     for (int jj = 0; jj < B_DMA; ++jj) {
-        const int row = 4 * (w + NW * jj) + (lane >> 4);
-        gB[jj] = Bg + (size_t)row * ldbB + (((lane & 15) ^ ((row & 7) << 1)) * 16);
+        if constexpr (ES == 1) {
+            const int row = 4 * (w + NW * jj) + (lane >> 4);
+            gB[jj] = Bg + (size_t)row * ldbB + (((lane & 15) ^ ((row & 7) << 1)) * 16);
+        } else {
+            const int row = 2 * (w + NW * jj) + (lane >> 5);
+            gB[jj] = Bg + (size_t)row * ldbB + (((lane & 31) ^ ((row & 3) << 2)) * 16);
+        }
     }
-    const size_t bStep = (size_t)64 * ldbB;
+    const size_t bStep = (size_t)(64 / ES) * ldbB;
     auto issue_b = [&](uint32_t ldsStage) {   // next k step of B
 #pragma unroll
         for (int jj = 0; jj < B_DMA; ++jj) {
@@ -166,23 +175,43 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0;
 
     // fragment addresses
-    // transpose read: within a 16-lane group, lane i supplies 8 bytes of k row (i>>1), column half (i&1)
+    // 1-byte transpose read: within a 16-lane group, lane i supplies 8 bytes of k row (i>>1), column half (i&1)
     // of a 16-column chunk, and receives column i of the chunk for 8 consecutive k rows.
-    const int ti16 = lane & 15, tch = (lane >> 4) & 1, trow = ti16 >> 1, thalf = ti16 & 1;
+    // 2-byte transpose read: lane i supplies 4 elements of k row (i>>2), column quad (i&3) of a 16-column (32-byte)
+    // chunk pair, and receives column i for 4 consecutive k rows.  Two reads make the 16 bytes of k a lane feeds
+    // the MFMA with; groups 0/1 of a half-wave take the two 16-column halves of a 32-column block, the upper
+    // half-wave the upper half of the k slab.
+    const int ti16 = lane & 15, tch = (lane >> 4) & 1;
     uint32_t b_lds[4];
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) {
-        const int q = wn * 8 + nb * 2 + tch;
-        b_lds[nb] = (16 * h + trow) * 256 + ((q ^ (2 * trow)) * 16) + thalf * 8;
+        if constexpr (ES == 1) {
+            const int trow = ti16 >> 1, thalf = ti16 & 1;
+            const int q = wn * 8 + nb * 2 + tch;
+            b_lds[nb] = (16 * h + trow) * 256 + ((q ^ (2 * trow)) * 16) + thalf * 8;
+        } else {
+            const int trow = ti16 >> 2, tq = ti16 & 3;
+            const int q = wn * 16 + nb * 4 + tch * 2 + (tq >> 1);
+            b_lds[nb] = (8 * h + trow) * 512 + ((q ^ (trow << 2)) * 16) + (tq & 1) * 8;
+        }
     }
+    constexpr int B_KK = (ES == 1) ? 32 * 256 : 16 * 512;     // bytes of a stage per 32-byte k slab
+    constexpr int B_HALF = (ES == 1) ? 8 * 256 : 4 * 512;     // second transpose read of a fragment
+    auto read_b1 = [&](v4i (&bf)[4], const unsigned char *sb, int kk, int nb) {
+        const unsigned char *p = sb + b_lds[nb] + kk * B_KK;
+        v2i t0, t1;
+        if constexpr (ES == 1) {
+            t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
+            t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + B_HALF));
+        } else {
+            t0 = __builtin_bit_cast(v2i, __builtin_amdgcn_ds_read_tr16_b64_v4i16((CATCOC_LDS v4s16 *)p));
+            t1 = __builtin_bit_cast(v2i, __builtin_amdgcn_ds_read_tr16_b64_v4i16((CATCOC_LDS v4s16 *)(p + B_HALF)));
+        }
+        bf[nb] = v4i{t0.x, t0.y, t1.x, t1.y};
+    };
     auto load_b = [&](v4i (&bf)[4], const unsigned char *sb, int kk) {
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-            const unsigned char *p = sb + b_lds[nb] + kk * 32 * 256;
-            const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
-            const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 256));
-            bf[nb] = v4i{t0.x, t0.y, t1.x, t1.y};
-        }
+        for (int nb = 0; nb < 4; ++nb) read_b1(bf, sb, kk, nb);
     };
     auto mma = [&](const v4i (&af)[MB], const v4i (&bf)[4]) {
 #pragma unroll
@@ -202,12 +231,6 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 #define CATCOC_MMA(FA, FB, MBI, NBI)                                              \
     acc[MBI][NBI] = mfma32<DT>(FA[MBI], FB[NBI], acc[MBI][NBI]);                  \
     CATCOC_FENCE();
-    auto read_b1 = [&](v4i (&bf)[4], const unsigned char *sb, int kk, int nb) {
-        const unsigned char *p = sb + b_lds[nb] + kk * 32 * 256;
-        const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
-        const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 256));
-        bf[nb] = v4i{t0.x, t0.y, t1.x, t1.y};
-    };
     // read_a(af, kk): A fragments of this step; sb: B stage of this step; slot1/2/3/4: the step's other work
     auto sched_step = [&](auto read_a, const unsigned char *sb, auto slot1, auto slot2, auto slot3, auto slot4) {
         CATCOC_MMA(fa1, fb1, 0, 0)
@@ -258,7 +281,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 #undef CATCOC_MMA
     auto nothing = [] {};
 
-    const uint32_t nk = args.K / 64;
+    const uint32_t nk = args.K * ES / 64;
     if constexpr (BM == 128) {
         // ---- 3 stages, copies run two k steps ahead (72 KiB LDS, two workgroups per CU) ----
         auto stA = [&](uint32_t s3) { return smem + s3 * A_STAGE; };
@@ -510,15 +533,32 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const uint32_t gcol0 = ti.col + col0;
     const uint32_t row_base = wm * 32 * MB + h * 4;
     const bool kept = ti.row >= args.keptBegin && ti.row < args.keptBegin + args.keptRows;
+    // W8A8 accumulators are dequantised in place (the registers then hold fp32 bit patterns); element accesses go
+    // through scalar temporaries
+    auto getf = [&](int mb, int nb, int r) -> float {
+        if constexpr (DT == DT_I8) {
+            const int iv = acc[mb][nb][r];
+            return i2f(iv);
+        } else {
+            const float fv = acc[mb][nb][r];
+            return fv;
+        }
+    };
+    auto setf = [&](int mb, int nb, int r, float v) {
+        if constexpr (DT == DT_I8) acc[mb][nb][r] = f2i(v);
+        else acc[mb][nb][r] = v;
+    };
 
-    if (args.bias != nullptr) {
+    if constexpr (DT == DT_I8) {
+        if (args.bias != nullptr) {
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-            const int bv = args.bias[gcol0 + 32 * nb];
+            for (int nb = 0; nb < 4; ++nb) {
+                const int bv = args.bias[gcol0 + 32 * nb];
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+                for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[mb][nb][r] += bv;
+                    for (int r = 0; r < 16; ++r) acc[mb][nb][r] += bv;
+            }
         }
     }
 
@@ -528,48 +568,58 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
-                int32_t *o = (int32_t *)args.accDump + (size_t)(ti.row + lrow) * args.N + gcol0;
-#pragma unroll
-                for (int nb = 0; nb < 4; ++nb) {
-                    const int iv = acc[mb][nb][r];
-                    o[32 * nb] = iv;
-                }
-            }
-    }
-
-    float sN[4];
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) sN[nb] = args.scaleN[gcol0 + 32 * nb];
-
-    if (kept) {
-        const uint32_t out_row0 = ti.row - args.keptBegin;
-        if (args.cAccum != nullptr) {
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
-                    int32_t *o = args.cAccum + (size_t)(out_row0 + lrow) * args.N + gcol0;
+                if constexpr (DT == DT_I8) {
+                    int32_t *o = (int32_t *)args.accDump + (size_t)(ti.row + lrow) * args.N + gcol0;
 #pragma unroll
                     for (int nb = 0; nb < 4; ++nb) {
                         const int iv = acc[mb][nb][r];
                         o[32 * nb] = iv;
                     }
-                }
-        }
-        // dequantise in place: per-channel scale first, then per-token, each product rounded on its own
+                } else {
+                    float *o = (float *)args.accDump + (size_t)(ti.row + lrow) * args.N + gcol0;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
-                const float sM = args.scaleM[ti.row + lrow];
-#pragma unroll
-                for (int nb = 0; nb < 4; ++nb) {
-                    const int iv = acc[mb][nb][r];
-                    acc[mb][nb][r] = f2i(__fmul_rn(__fmul_rn((float)iv, sN[nb]), sM));
+                    for (int nb = 0; nb < 4; ++nb) o[32 * nb] = getf(mb, nb, r);
                 }
             }
+    }
+
+    float sN[4] = {1.f, 1.f, 1.f, 1.f};
+    if constexpr (DT == DT_I8) {
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) sN[nb] = args.scaleN[gcol0 + 32 * nb];
+    }
+
+    if (kept) {
+        const uint32_t out_row0 = ti.row - args.keptBegin;
+        if constexpr (DT == DT_I8) {
+            if (args.cAccum != nullptr) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
+                        int32_t *o = args.cAccum + (size_t)(out_row0 + lrow) * args.N + gcol0;
+#pragma unroll
+                        for (int nb = 0; nb < 4; ++nb) {
+                            const int iv = acc[mb][nb][r];
+                            o[32 * nb] = iv;
+                        }
+                    }
+            }
+            // dequantise in place: per-channel scale first, then per-token, each product rounded on its own
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
+                    const float sM = args.scaleM[ti.row + lrow];
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb) {
+                        const int iv = acc[mb][nb][r];
+                        acc[mb][nb][r] = f2i(__fmul_rn(__fmul_rn((float)iv, sN[nb]), sM));
+                    }
+                }
+        }
 
         // one fp32 partial of the tile, added from global memory 32 rows (64 loads per lane) at a time
         // (device: the partial was written by other workgroups of this launch, read it at device scope)
@@ -590,10 +640,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
 #pragma unroll
-                    for (int nb = 0; nb < 4; ++nb) {
-                        const int iv = acc[mb][nb][r];
-                        acc[mb][nb][r] = f2i(__fadd_rn(i2f(iv), pv[r][nb]));
-                    }
+                    for (int nb = 0; nb < 4; ++nb) setf(mb, nb, r, __fadd_rn(getf(mb, nb, r), pv[r][nb]));
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -637,10 +684,8 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
                 for (int r = 0; r < 16; ++r) {
                     const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
 #pragma unroll
-                    for (int nb = 0; nb < 4; ++nb) {
-                        const int iv = acc[mb][nb][r];
-                        dptr[(size_t)lrow * args.ldd + 32 * nb] = (unsigned short)cvt(i2f(iv));
-                    }
+                    for (int nb = 0; nb < 4; ++nb)
+                        dptr[(size_t)lrow * args.ldd + 32 * nb] = (unsigned short)cvt(getf(mb, nb, r));
                 }
         };
         if (args.outDtype == DT_BF16) store_all([](float f) { return f32_to_bf16_bits(f); });
@@ -652,32 +697,42 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
-                const float sM = args.scaleM[ti.row + lrow];
+                if constexpr (DT == DT_I8) {
+                    const float sM = args.scaleM[ti.row + lrow];
 #pragma unroll
-                for (int nb = 0; nb < 4; ++nb) {
-                    const int iv = acc[mb][nb][r];
-                    __builtin_nontemporal_store(__fmul_rn(__fmul_rn((float)iv, sN[nb]), sM), ob + (size_t)lrow * sp.n0 + 32 * nb);
+                    for (int nb = 0; nb < 4; ++nb) {
+                        const int iv = acc[mb][nb][r];
+                        __builtin_nontemporal_store(__fmul_rn(__fmul_rn((float)iv, sN[nb]), sM), ob + (size_t)lrow * sp.n0 + 32 * nb);
+                    }
+                } else {
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb) __builtin_nontemporal_store(getf(mb, nb, r), ob + (size_t)lrow * sp.n0 + 32 * nb);
                 }
             }
     } else if (args.checksum != nullptr) {
-        long long *red = (long long *)smem;   // the pool is free again
-        long long si = 0;
+        // int64 sum of the int32 accumulators (W8A8) or double sum of the fp32 ones
+        using Sum = typename std::conditional<DT == DT_I8, long long, double>::type;
+        Sum *red = (Sum *)smem;   // the pool is free again
+        Sum si = 0;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) si += acc[mb][nb][r];
+                for (int r = 0; r < 16; ++r) {
+                    if constexpr (DT == DT_I8) si += acc[mb][nb][r];
+                    else si += (double)getf(mb, nb, r);
+                }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) si += __shfl_xor(si, o, 64);
         __syncthreads();   // every wave has left the main loop's LDS reads behind
         if (lane == 0) red[w] = si;
         __syncthreads();
         if (tid == 0) {
-            long long t = 0;
+            Sum t = 0;
 #pragma unroll
             for (int i = 0; i < NW; ++i) t += red[i];
-            ((long long *)args.checksum)[task] = t;
+            ((Sum *)args.checksum)[task] = t;
         }
     }
 

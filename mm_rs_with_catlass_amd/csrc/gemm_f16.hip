@@ -1,9 +1,21 @@
 // Instantiates the fused GEMM kernels for one element type.
+#include "gemm_dma_kernel.h"
 #include "gemm_fused_kernel.h"
 
 namespace catcoc {
 int launch_gemm_f16(const GemmArgs &args, int variant, bool edge, void *stream)
 {
     return launch_dt<DT_F16>(args, variant, edge, stream);
+}
+
+// Full-tile path with direct-to-LDS copies (row-major operands, see gemm_dma_kernel.h): m0 = 128 or 256.
+int launch_gemm_dma_f16(const GemmArgs &args, void *stream)
+{
+    const dim3 grid(args.sched.coreLoops);
+    if (args.sched.m0 == 256)
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_F16, 4, false>), grid, dim3(512), 0, (hipStream_t)stream, args);
+    else
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_F16, 2, false>), grid, dim3(256), 0, (hipStream_t)stream, args);
+    return (int)hipGetLastError();
 }
 }  // namespace catcoc

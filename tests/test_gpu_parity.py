@@ -365,6 +365,43 @@ def test_float_reduce_scatter(dtype, shape):
     assert np.abs(pd - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
 
 
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+def test_float_reduce_scatter_256_row_tiles_outbound_and_checksum(dtype):
+    # the direct-to-LDS kernel on 256x256 tiles; tiles of the other ranks checked through outbound stores / checksums
+    _need_gpu()
+    import ctypes as C
+    M, N, K, P, rank = 4096, 512, 320, 8, 6
+    rng = np.random.default_rng(21)
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    part, want = oracle.matmul_reduce(A, B, dtype, rank * rows, rows, peers, want_partial=True)
+    t = ops.default_tiling(M, K, N, P, m0=256, n0=256, k0=256)
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    so = L.load()
+    ntasks = so.catcoc_get_task_count(L.MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+    need = so.catcoc_get_workspace_size(L.MATMUL_REDUCE_SCATTER, L.FP16, C.byref(t), C.byref(d))
+    full = part[rank * rows:(rank + 1) * rows] + sum(peers)
+    for mode in ("checksum", "outbound"):
+        kw = {"checksum": torch.zeros(ntasks, dtype=torch.float64, device=DEV)} if mode == "checksum" else \
+             {"outbound": torch.zeros(need // 4, dtype=torch.float32, device=DEV)}
+        out = ops.matmul_reduce_scatter(dev16(A, dtype), dev16(B, dtype), [dev(p) for p in peers], rank, P, tiling=t, **kw)
+        torch.cuda.synchronize()
+        _check_float(host16(out), want, full, dtype, K)
+        tr, row, col, ws = (C.c_uint32() for _ in range(4))
+        for task in range(ntasks):
+            so.catcoc_task_tile(L.MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row), C.byref(col), C.byref(ws))
+            blk = part[row.value:row.value + 256, col.value:col.value + 256]
+            if mode == "checksum":
+                got = float(kw["checksum"][task])
+                want_cs = 0.0 if tr.value == rank else float(blk.astype(np.float64).sum())
+                assert abs(got - want_cs) <= 1e-2 * max(1.0, np.abs(blk).sum()), task
+            elif tr.value != rank:
+                ob = kw["outbound"].cpu().numpy().reshape(-1, 256)[ws.value:ws.value + 256]
+                assert np.abs(ob - blk).max() <= 1e-2 * max(1.0, np.abs(blk).max()), task
+
+
 def test_float_allreduce_config1_full_size():
     # BASELINE config 1: A[512,2048], B[2048,1024] fp16 ~U(-1,1), K halves as the two ranks' partials
     _need_gpu()
