@@ -9,6 +9,7 @@ in HBM before the timed region.  Prints ONE JSON line.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode kept|outbound] [--no-cpu]
     python bench.py --mode copy     # plain 256 MiB device copy: the known-size kernel the HBM counters are scaled by
     python bench.py --mode decode   # BASELINE config 5: skinny-M sweep, K = N = 8192, GB/s per M (HBM-bound)
+    python bench.py --mode float    # BASELINE configs 3 (fp16 reduce-scatter), 2 (bf16 all-gather) and 1 (fp16 all-reduce)
 """
 import argparse
 import json
@@ -106,12 +107,81 @@ def decode_sweep(args, torch, L, ops, dev):
         "sweep": sweep}))
 
 
+PEAK_F16_TFLOPS = 2500.0   # MI355X dense fp16 / bf16 MFMA, published
+
+
+def float_configs(args, torch, L, ops, dev):
+    """BASELINE configs 3, 2 and 1 (float GEMMs with fp32 accumulate); value = config 3."""
+    import numpy as np
+    import oracle
+    g = torch.Generator(device=dev).manual_seed(20250101)
+
+    def timed(fn):
+        fn()
+        L.check()
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps, e0.elapsed_time(e1) / args.steps / 1e3
+
+    res = []
+    # config 3: fp16 matmul-reduce-scatter, A[4096,1792] N(0,1), B[1792,4096] N(0,0.02), 7 fp32 peers, keep [512,4096]
+    M, K, N, P, rank = 4096, 1792, 4096, 8, 0
+    rows = M // P
+    A = torch.randn((M, K), device=dev, generator=g).half()
+    B = (torch.randn((K, N), device=dev, generator=g) * 0.02).half()
+    peers = [torch.randn((rows, N), device=dev, generator=g) for _ in range(P - 1)]
+    cs = torch.zeros(4096, dtype=torch.float64, device=dev)
+    out = torch.empty((rows, N), dtype=torch.float16, device=dev)
+    wall, kern = timed(lambda: ops.matmul_reduce_scatter(A, B, peers, rank, P, checksum=cs, out=out))
+    sel = np.arange(0, rows, 61)
+    _, want = oracle.matmul_reduce(A[sel].view(torch.int16).cpu().numpy().view(np.uint16), B.view(torch.int16).cpu().numpy().view(np.uint16),
+                                   oracle.FP16, 0, len(sel), [p[sel].cpu().numpy() for p in peers])
+    got = out[sel].view(torch.int16).cpu().numpy().view(np.uint16)
+    rel = float(np.abs(got.view(np.float16).astype(np.float32) - want.view(np.float16).astype(np.float32)).max())
+    res.append({"config": 3, "op": "matmul_reduce_scatter fp16 M=4096 K=1792 N=4096 P=8", "kernel_us": round(kern * 1e6, 2),
+                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * M * N * K / kern / 1e12, 1), "max_abs_err_sample": rel})
+    # config 2: bf16 all-gather matmul, 8 shards [512,4096], B[4096,1024]
+    m, K, N, P = 512, 4096, 1024, 8
+    shards = [torch.randn((m, K), device=dev, generator=g).bfloat16() for _ in range(P)]
+    B2 = (torch.randn((K, N), device=dev, generator=g) * 0.02).bfloat16()
+    out2 = torch.empty((m * P, N), dtype=torch.bfloat16, device=dev)
+    wall, kern = timed(lambda: ops.allgather_matmul(shards[0], shards[1:], B2, 0, P, out=out2))
+    res.append({"config": 2, "op": "allgather_matmul bf16 8 x [512,4096] x [4096,1024]", "kernel_us": round(kern * 1e6, 2),
+                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * m * P * N * K / kern / 1e12, 1)})
+    # config 1: fp16 all-reduce share, A[512,1024] (this rank's k half), B[1024,1024], one fp32 peer
+    M, K, N, P = 512, 1024, 1024, 2
+    A1 = (torch.rand((M, K), device=dev, generator=g) * 2 - 1).half()
+    B1 = (torch.rand((K, N), device=dev, generator=g) * 2 - 1).half()
+    peer = [torch.randn((M, N), device=dev, generator=g)]
+    out1 = torch.empty((M, N), dtype=torch.float16, device=dev)
+    wall, kern = timed(lambda: ops.matmul_allreduce(A1, B1, peer, 0, P, out=out1))
+    res.append({"config": 1, "op": "matmul_allreduce fp16 M=512 K=1024(local) N=1024 P=2", "kernel_us": round(kern * 1e6, 2),
+                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * M * N * K / kern / 1e12, 1)})
+    c3 = res[0]
+    print(json.dumps({
+        "metric": "fp16 matmul-reduce-scatter shard (BASELINE config 3) TFLOPS, 1 MI355X", "value": c3["TFLOPS"], "unit": "TFLOPS",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": c3["wall_us"] / 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": c3["op"] + ", 7 staged fp32 peers, fp16 [512,4096] kept"},
+        "roofline": {"bound": "mfma", "achieved": c3["TFLOPS"], "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(c3["TFLOPS"] / PEAK_F16_TFLOPS, 4), "traffic": None},
+        "configs": res}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode"], default="kept",
+    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode", "float"], default="kept",
                     help="kept: non-kept tiles are folded into checksums (BASELINE's literal outputs); "
                          "outbound: they are also stored as fp32 to the symmetric workspace")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -150,6 +220,9 @@ def main():
         return
     if args.mode == "decode":
         decode_sweep(args, torch, L, ops, dev)
+        return
+    if args.mode == "float":
+        float_configs(args, torch, L, ops, dev)
         return
     M, K, N, P, rank = 8192, 1792, 4096, 8, args.rank
     rows = M // P
