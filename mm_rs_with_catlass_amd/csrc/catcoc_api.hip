@@ -237,7 +237,7 @@ void launch_float(int commType, int dataType, void *stream, uint8_t *a, uint8_t 
     p.args.b = b;
     p.args.d = c;
     if (!check_ptr_align(p, a, b)) p.variant = 0;
-    const bool dma = p.dma && p.variant != 0 && (uintptr_t)b % 16 == 0 && (p.args.ldb * 2) % 16 == 0;
+    const bool dma = p.dma && p.variant != 0 && (uintptr_t)b % 16 == 0 && (p.args.ldb * 2) % 16 == 0 && (uintptr_t)c % 16 == 0;
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles and 16-byte aligned row-major operands"); return; }
     const int e = dma ? (p.dtype == DT_F16 ? launch_gemm_dma_f16(p.args, stream) : launch_gemm_dma_bf16(p.args, stream))
                       : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
@@ -368,7 +368,7 @@ void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uin
     if (!check_ptr_align(p, x1, x2) || (uintptr_t)scale_x2 % 16 != 0 || (bias && (uintptr_t)bias % 16 != 0) ||
         (c_accum && (uintptr_t)c_accum % 16 != 0) || (uintptr_t)d_out % 8 != 0)
         p.variant = 0;
-    bool dma = p.dma && p.variant != 0 && (uintptr_t)x2 % 16 == 0 && p.args.ldb % 16 == 0;
+    bool dma = p.dma && p.variant != 0 && (uintptr_t)x2 % 16 == 0 && p.args.ldb % 16 == 0 && (uintptr_t)d_out % 16 == 0;
     for (uint32_t s = 0; s < p.args.nPeers && dma; ++s) dma = (uintptr_t)p.args.peers[s] % 16 == 0;
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles, 16-byte aligned row-major operands and fp32 peers"); return; }
     if (p.args.presum && (p.args.peerLd % 4 != 0)) p.args.presum = nullptr;

@@ -676,20 +676,34 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             }
         }
 
-        unsigned short *dptr = (unsigned short *)args.d + (size_t)out_row0 * args.ldd + gcol0;
-        auto store_all = [&](auto cvt) {
+        // 16-bit output.  A lane holds single columns 32 apart, so storing from registers would write 64-byte
+        // pieces (half a cache line each, 128 store instructions per lane).  Instead every wave turns its 64 x 128
+        // block around in a private 16 KiB LDS area: 2-byte writes in accumulator layout, 16-byte reads along the
+        // rows, and 16 stores per lane that each cover four whole 256-byte row segments.  Rows with bit 2 set
+        // (the upper half-wave of a write) are shifted by 128 bytes, which keeps both half-waves on different banks.
+        static_assert(NW * 16384 <= POOL, "one 16 KiB staging area per wave");
+        unsigned char *st = smem + w * 16384;
+        __syncthreads();   // every wave has left the main loop's LDS reads behind
+        auto stage_all = [&](auto cvt) {
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
+                    const uint32_t wrow = mb * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
 #pragma unroll
                     for (int nb = 0; nb < 4; ++nb)
-                        dptr[(size_t)lrow * args.ldd + 32 * nb] = (unsigned short)cvt(getf(mb, nb, r));
+                        *(unsigned short *)(st + wrow * 256 + (((nb * 32 + c32) * 2) ^ (h << 7))) = (unsigned short)cvt(getf(mb, nb, r));
                 }
         };
-        if (args.outDtype == DT_BF16) store_all([](float f) { return f32_to_bf16_bits(f); });
-        else store_all([](float f) { return f32_to_f16_bits(f); });
+        if (args.outDtype == DT_BF16) stage_all([](float f) { return f32_to_bf16_bits(f); });
+        else stage_all([](float f) { return f32_to_f16_bits(f); });
+        unsigned char *dwave = (unsigned char *)args.d + ((size_t)(out_row0 + wm * 32 * MB) * args.ldd + ti.col + wn * 128) * 2;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const uint32_t wrow = j * 4 + (lane >> 4), chunk = lane & 15;
+            const v4i v = *(const v4i *)(st + wrow * 256 + ((chunk * 16) ^ (((wrow >> 2) & 1) << 7)));
+            *(v4i *)(dwave + (size_t)wrow * args.ldd * 2 + chunk * 16) = v;
+        }
     } else if (args.flags & GF_OUTBOUND_STORE) {
         float *ob = (float *)args.outbound + (size_t)ti.wsRow * sp.n0 + col0;
 #pragma unroll
