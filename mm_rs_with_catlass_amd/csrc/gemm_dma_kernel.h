@@ -583,10 +583,20 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             }
     }
 
+    // W8A8 scales of this lane's rows and columns, fetched in one batch (32 + 4 loads in flight together;
+    // fetched one row at a time next to their use they cost a memory round trip per row)
     float sN[4] = {1.f, 1.f, 1.f, 1.f};
+    float sMv[MB][16];
     if constexpr (DT == DT_I8) {
+        if (kept || (args.flags & GF_OUTBOUND_STORE)) {
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) sN[nb] = args.scaleN[gcol0 + 32 * nb];
+            for (int nb = 0; nb < 4; ++nb) sN[nb] = args.scaleN[gcol0 + 32 * nb];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sMv[mb][r] = args.scaleM[ti.row + row_base + mb * 32 + (r >> 2) * 8 + (r & 3)];
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 
     if (kept) {
@@ -611,8 +621,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
-                    const float sM = args.scaleM[ti.row + lrow];
+                    const float sM = sMv[mb][r];
 #pragma unroll
                     for (int nb = 0; nb < 4; ++nb) {
                         const int iv = acc[mb][nb][r];
@@ -712,7 +721,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             for (int r = 0; r < 16; ++r) {
                 const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
                 if constexpr (DT == DT_I8) {
-                    const float sM = args.scaleM[ti.row + lrow];
+                    const float sM = sMv[mb][r];
 #pragma unroll
                     for (int nb = 0; nb < 4; ++nb) {
                         const int iv = acc[mb][nb][r];
