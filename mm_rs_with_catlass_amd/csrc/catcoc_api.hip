@@ -537,9 +537,8 @@ uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const C
     ok();
     const SchedParams &s = p.args.sched;
     if (wg >= s.coreLoops) return 0xffffffffu;
-    const bool linear = (p.args.flags & GF_LINEAR_ORDER) != 0;
-    const uint32_t seq = launch_seq(s, wg, linear);
-    return linear ? seq : kept_order_task(s, p.args.keptRank, seq, p.args.presum != nullptr);
+    if (!p.dma) return launch_order_task(s, wg, (p.args.flags & GF_LINEAR_ORDER) != 0, p.args.keptRank);
+    return launch_task(s, wg, (p.args.flags & GF_LINEAR_ORDER) != 0, p.args.keptRank, p.args.presum != nullptr);
 }
 
 uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags)

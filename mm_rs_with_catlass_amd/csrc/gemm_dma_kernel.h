@@ -116,7 +116,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const bool linear = (args.flags & GF_LINEAR_ORDER) != 0;
     const bool presum = PRESUM && args.presum != nullptr;
     const uint32_t seq = launch_seq(sp, blockIdx.x, linear);
-    const uint32_t task = linear ? seq : kept_order_task(sp, args.keptRank, seq, presum);
+    const uint32_t task = launch_task(sp, blockIdx.x, linear, args.keptRank, presum);
     TileInfo ti;
     if (!task_tile(sp, task, ti)) return;
 

@@ -42,6 +42,21 @@ CATCOC_HD void swizzle_block_coord(uint32_t off, uint32_t dir, uint32_t loopsM, 
     else banded_walk(off, loopsN, loopsM, inner, true, nIdx, mIdx);
 }
 
+// Inverse of banded_walk / swizzle_block_coord: the position of tile (mIdx, nIdx) in the swizzled order.
+CATCOC_HD uint32_t banded_index(uint32_t width, uint32_t lenBanded, uint32_t lenOther, bool serpentine, uint32_t posBanded,
+                                uint32_t posOther)
+{
+    const uint32_t band = posBanded / width;
+    const uint32_t w = umin(width, lenBanded - band * width);
+    const uint32_t q = (serpentine && (band & 1u)) ? lenOther - 1u - posOther : posOther;
+    return band * width * lenOther + q * w + (posBanded - band * width);
+}
+
+CATCOC_HD uint32_t swizzle_block_index(uint32_t off, uint32_t dir, uint32_t loopsM, uint32_t loopsN, uint32_t mIdx, uint32_t nIdx)
+{
+    return dir == 0 ? banded_index(off, loopsM, loopsN, true, mIdx, nIdx) : banded_index(off, loopsN, loopsM, true, nIdx, mIdx);
+}
+
 // SplitkGemmIdentityBlockSwizzle (block_swizzle.hpp:151-158): first k tile of slice s.
 CATCOC_HD uint32_t splitk_first_ktile(uint32_t kTiles, uint32_t f, uint32_t s)
 {
@@ -248,6 +263,66 @@ CATCOC_HD uint32_t kept_order_task(const SchedParams &s, uint32_t keptRank, uint
 
 // Position of a workgroup in the launch sequence (XCD-aware chunking).
 CATCOC_HD uint32_t launch_seq(const SchedParams &s, uint32_t wg, bool linear) { return workgroup_task(wg, s.coreLoops, linear); }
+
+// XCD-block launch order for reduce-scatter and all-reduce launches.  Consecutive workgroups go round-robin to the
+// 8 XCDs, each with its own L2, so XCD x = wg mod 8 is given one block of the global tile grid (all ranks' rows):
+// the grid is cut RX x CX = 8 ways, rows dealt round-robin to the RX row parts (every part then holds the same share
+// of each rank's rows, kept ones included) and columns cut into CX contiguous parts, with RX x CX chosen to minimise
+// the A rows plus B columns one XCD touches.  Inside its block an XCD walks row by row with the kept rank's rows
+// first, so the tiles in flight on an XCD at any time share a few A row blocks and all of the block's B columns.
+// Returns false when the grid does not divide evenly (callers fall back to the chunked order).
+CATCOC_HD bool xcd_block_task(const SchedParams &s, uint32_t keptRank, uint32_t wg, uint32_t &task)
+{
+    if (s.op == OP_ALLGATHER || (s.coreLoops & 7u) != 0 || wg >= s.coreLoops) return false;
+    const bool rs = s.op == OP_REDUCE_SCATTER;
+    const uint32_t GM = (rs ? s.P : 1u) * s.loopsM;
+    if (GM * s.loopsN != s.coreLoops) return false;
+    uint32_t RX = 0, best = 0xffffffffu;
+    for (uint32_t r = 1; r <= 8; r <<= 1) {
+        const uint32_t c = 8u / r;
+        if (GM % r != 0 || s.loopsN % c != 0) continue;
+        const uint32_t cost = (GM / r) * s.m0 + (s.loopsN / c) * s.n0;
+        if (cost < best) { best = cost; RX = r; }
+    }
+    if (RX == 0) return false;
+    const uint32_t CX = 8u / RX, rowsPer = GM / RX, colsPer = s.loopsN / CX;
+    const uint32_t x = wg & 7u, j = wg >> 3;
+    const uint32_t rp = x / CX, cp = x - rp * CX;
+    const uint32_t ri = j / colsPer, ci = j - ri * colsPer;
+    // rows of this part are rp + RX*i; those of the kept rank are i in [i0, i1)
+    uint32_t i0 = 0, i1 = 0;
+    if (rs && s.P > 1) {
+        const uint32_t lo = keptRank * s.loopsM, hi = lo + s.loopsM;
+        i0 = lo > rp ? ceil_div(lo - rp, RX) : 0u;
+        i1 = hi > rp ? ceil_div(hi - rp, RX) : 0u;
+        i0 = umin(i0, rowsPer);
+        i1 = umin(i1, rowsPer);
+    }
+    const uint32_t nk = i1 - i0;
+    uint32_t i;
+    if (ri < nk) i = i0 + ri;
+    else { const uint32_t t = ri - nk; i = t < i0 ? t : t + nk; }
+    const uint32_t gr = rp + RX * i, nIdx = cp * colsPer + ci;
+    const uint32_t rank = gr / s.loopsM, mIdx = gr - rank * s.loopsM;
+    const uint32_t inRank = swizzle_block_index(s.off, s.dir, s.loopsM, s.loopsN, mIdx, nIdx);
+    if (!rs) { task = inRank; return true; }
+    const uint32_t perRank = s.blockPerComm / s.P;
+    const uint32_t round = inRank / perRank, idx = inRank - round * perRank;
+    const uint32_t commLoops = ceil_div(s.coreLoops, s.blockPerComm);
+    const uint32_t actual = (round == commLoops - 1u) ? s.coreLoops - round * s.blockPerComm : s.blockPerComm;
+    task = round * s.blockPerComm + rank * (actual / s.P) + idx;
+    return true;
+}
+
+// Workgroup -> task of a launch: the XCD-block order where it applies, else XCD-aware chunking with the kept
+// rank's tiles first (last when the other tiles pre-sum the peers for them).
+CATCOC_HD uint32_t launch_task(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank, bool keptLast)
+{
+    if (linear) return wg;
+    uint32_t task;
+    if (!keptLast && xcd_block_task(s, keptRank, wg, task)) return task;
+    return kept_order_task(s, keptRank, workgroup_task(wg, s.coreLoops, false), keptLast);
+}
 
 // Workgroup -> task of a launch: XCD-aware chunking, then kept-first ordering.
 CATCOC_HD uint32_t launch_order_task(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank)
