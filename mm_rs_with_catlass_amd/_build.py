@@ -7,6 +7,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
 LIB = os.path.join(PKG, "libcatcoc_hip.so")
+HOST_EXAMPLE = os.path.join(PKG, "catcoc_quant_rs_host")   # C++ host driving the library through its C ABI alone
 OBJ_DIR = os.path.join(PKG, "csrc", "build")
 
 HIPCC_FLAGS = [
@@ -46,6 +47,14 @@ def build(verbose=False, extra=(), jobs=8):
     # runtime in one process cannot open the device).
     cxx = os.environ.get("CXX", "g++")
     cmd = [cxx, "-shared", "-fPIC", *objs, "-o", LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    # the stand-alone C++ host: plain g++, links the HIP runtime itself and the library beside it
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [cxx, "-O2", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"), "-I", os.path.join(rocm, "include"),
+           os.path.join(PKG, "csrc", "host_quant_rs.cpp"), "-o", HOST_EXAMPLE, "-L", PKG, "-lcatcoc_hip",
+           "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(rocm, "lib")]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)

@@ -490,3 +490,37 @@ def test_quant_config4_full_size_properties():
     blk = dump[rank * rows:(rank + 1) * rows].float()
     want0 = ((blk * s2[None, :]) * s1[rank * rows:(rank + 1) * rows, None]).to(torch.bfloat16)
     assert torch.equal(out0.view(torch.int16), want0.view(torch.int16))
+
+
+# ------------------------------------------------------- C ABI from a plain C++ host
+def test_cpp_host_drives_the_library_through_the_c_abi(tmp_path):
+    # the stand-alone host (no Python, no torch in the process) reads the reference's raw .bin files, launches
+    # catcoc_quant_matmul_reduce_scatter and writes this rank's block of output.bin at its offset
+    _need_gpu()
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(L.LIB_PATH), "catcoc_quant_rs_host")
+    assert os.path.exists(exe), "build the package first (python -m mm_rs_with_catlass_amd._build)"
+    M, N, K, P, rank = 1024, 512, 256, 4, 2
+    rng = np.random.default_rng(77)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.integers(-1000, 1000, N, dtype=np.int32)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    for name, arr in (("x1_gm", x1), ("x2_gm", x2), ("scale_x1_gm", s1), ("scale_x2_gm", s2), ("bias_gm", b)):
+        arr.tofile(tmp_path / (name + ".bin"))
+    for i, p in enumerate(peers):
+        p.tofile(tmp_path / ("peer_%d.bin" % i))
+    r = subprocess.run([exe, str(P), str(rank), str(M), str(N), str(K), str(tmp_path)], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stderr + r.stdout
+    _, want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, b, rank * rows, rows, peers, oracle.BF16, want_acc=False)
+    got = np.fromfile(tmp_path / "output.bin", dtype=np.uint16)
+    assert got.size == (rank + 1) * rows * N
+    assert np.array_equal(got[rank * rows * N:].reshape(rows, N), want)
+    assert not got[:rank * rows * N].any()
+    # a rejected launch is reported, not executed
+    r = subprocess.run([exe, str(P), str(rank), str(M), str(N), str(K), str(tmp_path / "missing")], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 1 and "cannot read" in r.stderr
