@@ -119,6 +119,10 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const uint32_t task = launch_task(sp, blockIdx.x, linear, args.keptRank, presum);
     TileInfo ti;
     if (!task_tile(sp, task, ti)) return;
+    // The kept tiles are the longest chain of a reduce-scatter launch (main loop, then the peers' partials):
+    // their waves get priority over the other workgroup on the CU so that the chain starts its streaming early.
+    if (sp.op == OP_REDUCE_SCATTER && sp.P > 1 && ti.row >= args.keptBegin && ti.row < args.keptBegin + args.keptRows)
+        __builtin_amdgcn_s_setprio(3);
 
     const int64_t ldaB = args.lda * ES, ldbB = args.ldb * ES;  // row pitches in bytes
     const bool gather = sp.op == OP_ALLGATHER;
