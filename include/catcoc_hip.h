@@ -114,8 +114,6 @@ typedef struct CatcocSymmetricDesc {
     uint32_t keptRows;        /* keptRows != 0 (W8A8 only): the rank keeps rows [keptRowBegin, +keptRows) of an m that need not
                                  divide by rankSize, and the launch takes the skinny-M split-K path (decode shapes) */
     uint32_t splitK;          /* split-K path: k slices per tile; 0 = GetSplitkFactor with blockNum cores and 128x128x256 tiles */
-    uint32_t reduceWaitPolls; /* pre-sum path: polls (about 1 us apart) a kept tile waits for the workspace sum before it
-                                 adds the peers itself; 0 = 100000, 1 = do not wait at all */
     /* Reduce paths: peers[s], s = 0..rankSize-2, are the other ranks' partial
      * results for this rank's kept rows (fp32, or int32 with REDUCE_INT32), added
      * in slot order after the local partial.  Row `peerRowOffset + i` of a peer
@@ -129,14 +127,9 @@ typedef struct CatcocSymmetricDesc {
     uint64_t outboundBytes;   /* capacity of `outbound` */
     int64_t *checksum;        /* OUTBOUND_CHECKSUM target: one int64 per task (W8A8) / one double per task (float) */
     void *accDump;            /* optional full [m,n] int32 (W8A8) or fp32 (float) local partial, for bit-exact checks */
-    /* Optional scratch in HBM, catcoc_get_reduce_workspace_size() bytes, 256-byte aligned, ZEROED by the caller
-     * once before its first use (the library leaves it re-armed after every launch).  With it a W8A8
-     * reduce-scatter launch on 256x256 tiles lets the workgroups of the other ranks' tiles add up the peers'
-     * partials (p0 + p1 + ... in slot order) while they compute, and the kept tiles add that one sum:
-     * d = local + (p0 + p1 + ...) instead of ((local + p0) + p1) + ..., within one output ulp of each other.
-     * Launches that share a workspace must not overlap (same stream, or ordered by events).
-     * The split-K path keeps its int32 partial tiles and tile counters here instead
-     * (catcoc_get_splitk_workspace_size() bytes, same rules). */
+    /* Split-K path only: int32 partial tiles and tile counters, catcoc_get_splitk_workspace_size() bytes,
+     * 256-byte aligned, ZEROED by the caller once before its first use (the library leaves it re-armed after
+     * every launch).  Launches that share a workspace must not overlap (same stream, or ordered by events). */
     void *workspace;
     uint64_t workspaceBytes;
 } CatcocSymmetricDesc;
@@ -209,12 +202,6 @@ CATCOC_API int catcoc_can_implement(int commType, int dataType, const CocTilingP
 CATCOC_API uint64_t catcoc_get_workspace_size(int commType, int dataType, const CocTilingParams *tiling,
                                               const CatcocSymmetricDesc *desc);
 
-/* Bytes of `workspace` with which this W8A8 reduce-scatter launch would pre-sum the peers' partials
- * (fp32 [m/rankSize, n] + 256 control bytes); 0 when the shape does not qualify (it needs 256x256
- * tiles: m/rankSize and n multiples of 256, k a multiple of 128, row-major operands, fp32 peers, at most
- * 128 kept tiles).  No counterpart in the reference, whose reduce runs on separate vector cores. */
-CATCOC_API uint64_t catcoc_get_reduce_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc);
-
 /* Split-K path (descriptor with keptRows != 0): bytes of `workspace` the launch needs (0 when the split factor
  * is 1), the split factor it will use and its number of 128x128 tiles (`checksum`, if given, needs one int64 per
  * tile and receives the sum of the accumulators of the tile's rows that are not kept).  The path takes row-major
@@ -274,8 +261,8 @@ CATCOC_API void catcoc_comm_block_idx(uint32_t dir, uint32_t P, uint32_t splitRo
 CATCOC_API int catcoc_task_tile(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
                                 uint32_t task, uint32_t *targetRank, uint32_t *row, uint32_t *col,
                                 uint32_t *wsRow);
-/* The task workgroup `wg` of a launch runs: XCD-aware chunking, then the kept rank's tiles first (they are the
- * long ones), or last when the descriptor carries a pre-sum workspace.  A bijection on [0, task count);
+/* The task workgroup `wg` of a launch runs: an XCD-aware order with the kept rank's tiles first (they are the
+ * long ones).  A bijection on [0, task count);
  * 0xffffffff for wg out of range or rejected arguments.  No counterpart in the reference, where AI core i
  * simply runs tasks i, i + BLOCK_NUM, ... (quant_matmul_reduce_scatter.hpp:166-170). */
 CATCOC_API uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,

@@ -65,7 +65,6 @@ struct Plan {
     uint32_t dtype;
     uint32_t blockNum;
     bool dma;     // full tiles, row-major operands: the direct-to-LDS kernel applies
-    uint64_t presumBytes;  // workspace with which this launch would pre-sum the peers (0 = shape does not qualify)
 };
 
 uint32_t elem_size(uint32_t dt) { return dt == DT_I8 ? 1u : 2u; }
@@ -111,14 +110,7 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     if (n0 == 0) n0 = 256;
     const bool can256 = n0 == 256 && !transA && !transB && mRank % 256 == 0 && t->n % 256 == 0 &&
                         ((uint64_t)t->k * es) % 128 == 0 && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
-    // the peer pre-sum needs 256-row tiles, few enough kept tiles to be resident together, and other tiles to do it
-    const uint32_t tiles256 = can256 ? (t->m / 256) * (t->n / 256) : 0;
-    const bool presumShape = can256 && dt == DT_I8 && op == OP_REDUCE_SCATTER && P > 1 && !(d->flags & CATCOC_FLAG_LINEAR_ORDER) &&
-                             tiles256 / P <= 128 && (t->m0 == 0 || t->m0 == 256);
-    plan.presumBytes = presumShape ? (uint64_t)mRank * t->n * 4u + 256u : 0;
-    const bool presum = presumShape && d->workspace != nullptr;
-    // measured on MI355X: two 128x256 workgroups per CU beat one 256x256 workgroup at every k tried
-    if (m0 == 0) m0 = presum ? 256 : (mRank <= 64) ? 64 : 128;
+    if (m0 == 0) m0 = (mRank <= 64) ? 64 : 128;
     const bool dmaShape = can256 && m0 == 256;
     const bool fastShape = dmaShape || n0 == 256 && (m0 == 64 || m0 == 128) && !transA && t->k % che == 0 && t->n % 4 == 0;
     plan.variant = fastShape ? (int)(m0 / 64) : 0;   // 4 (m0 = 256) exists only as the direct-to-LDS kernel
@@ -197,19 +189,6 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
         a.checksum = d->checksum;
     }
     a.accDump = d->accDump;
-
-    if (presum && m0 == 256) {
-        if ((uintptr_t)d->workspace % 256 != 0) return fail(E_WORKSPACE, "workspace must be 256-byte aligned");
-        if (d->workspaceBytes < plan.presumBytes)
-            return fail(E_WORKSPACE, "workspace too small for the peer pre-sum: %llu < %llu bytes",
-                        (unsigned long long)d->workspaceBytes, (unsigned long long)plan.presumBytes);
-        a.presum = (float *)d->workspace;
-        a.presumCtl = (uint32_t *)((unsigned char *)d->workspace + (uint64_t)mRank * t->n * 4u);
-        a.keptTiles = a.sched.coreLoops / P;
-        a.presumProducers = a.sched.coreLoops - a.keptTiles;
-        a.presumUnits = (uint32_t)(((uint64_t)mRank * t->n * 4u) / 8192u);
-        a.presumSpin = (d->reduceWaitPolls ? d->reduceWaitPolls : 100001u) - 1u;
-    }
     return 0;
 }
 
@@ -371,7 +350,6 @@ void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uin
     bool dma = p.dma && p.variant != 0 && (uintptr_t)x2 % 16 == 0 && p.args.ldb % 16 == 0 && (uintptr_t)d_out % 16 == 0;
     for (uint32_t s = 0; s < p.args.nPeers && dma; ++s) dma = (uintptr_t)p.args.peers[s] % 16 == 0;
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles, 16-byte aligned row-major operands and fp32 peers"); return; }
-    if (p.args.presum && (p.args.peerLd % 4 != 0)) p.args.presum = nullptr;
     const int e = dma ? launch_gemm_dma_i8(p.args, stream) : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
     ok();
@@ -460,20 +438,6 @@ uint64_t catcoc_get_workspace_size(int commType, int dataType, const CocTilingPa
     return (uint64_t)p.args.sched.stages * p.args.sched.blockPerComm * p.args.sched.m0 * p.args.sched.n0 * 4u;
 }
 
-uint64_t catcoc_get_reduce_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc)
-{
-    Plan p;
-    CatcocSymmetricDesc d;
-    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
-    d = *desc;
-    d.flags &= ~CATCOC_OUTBOUND_MASK;
-    d.workspace = nullptr;
-    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
-    if (make_plan(QUANT_MATMUL_REDUCE_SCATTER, INT8, tiling, &d, 0, 0, p)) return 0;
-    ok();
-    return p.presumBytes;
-}
-
 uint64_t catcoc_get_splitk_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t *splitK,
                                           uint32_t *tiles)
 {
@@ -538,7 +502,7 @@ uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const C
     const SchedParams &s = p.args.sched;
     if (wg >= s.coreLoops) return 0xffffffffu;
     if (!p.dma) return launch_order_task(s, wg, (p.args.flags & GF_LINEAR_ORDER) != 0, p.args.keptRank);
-    return launch_task(s, wg, (p.args.flags & GF_LINEAR_ORDER) != 0, p.args.keptRank, p.args.presum != nullptr);
+    return launch_task(s, wg, (p.args.flags & GF_LINEAR_ORDER) != 0, p.args.keptRank);
 }
 
 uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags)

@@ -38,14 +38,6 @@ struct GemmArgs {
     uint32_t flags;                // GF_*
     uint32_t outDtype;             // DT_F16 / DT_BF16
     uint32_t transA, transB;
-    // Peer pre-sum of a reduce-scatter launch (NULL = off): S[keptRows, N] fp32 = sum of the peers' partials,
-    // produced by the first presumProducers workgroups of the launch sequence, consumed by the kept tiles.
-    float *presum;
-    uint32_t *presumCtl;           // [0] producers whose part of S is complete, [1] workgroups that have finished
-    uint32_t presumProducers;
-    uint32_t presumUnits;          // S in units of 8 KiB
-    uint32_t presumSpin;           // polls (about a microsecond apart) before a kept tile adds the peers itself
-    uint32_t keptTiles;
     // Skinny-M split-K launch: k slices per tile, int32 partial tiles [splitK][tiles][128][128], one counter per tile.
     uint32_t splitK;
     int32_t *skPart;

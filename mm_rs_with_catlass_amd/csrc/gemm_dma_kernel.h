@@ -4,16 +4,17 @@
 // transpose-read instruction, so the main loop issues almost nothing but LDS reads
 // and MFMAs.
 //
-// Reduce-scatter launches have few kept tiles, and streaming the peers' partials for
-// them on a few CUs is slow (a CU sustains a small share of the HBM bandwidth).  With
-// PRESUM the NON-kept workgroups each add up a slice of the peers' partials while
-// their own main loop runs: one extra 1 KiB copy per wave per k step into a small LDS
-// ring, summed in registers and written to a scratch buffer S = p0 + p1 + ...  The
-// kept tiles run last, wait for a counter that says S is complete, and add S instead
-// of the individual peers.
-//
-// Same per-tile contract as gemm_fused_kernel (see gemm_fused_kernel.h); used when
-// every tile is full, A is [rows,K] and B is [K,N], both row-major.
+// Reduce-scatter launches have few kept tiles, and each of them has to add the peers'
+// partials for its rows (0.9 MB per tile at 128x256 with 7 peers), which takes longer
+// than the tile's main loop and keeps its slot on the CU busy while the rest of the
+// launch runs out of work to pack around it.  With a workspace the kept tiles only
+// publish their dequantised fp32 tile and leave; the workgroups of the second half of
+// the launch each add the peers for one slice of the kept block after their own tile,
+// in the same order per element (local, then peers in slot order), so the result is
+// bit-identical and the reduce work is spread evenly over every slot.  A slice is
+// finished on the XCD that published it: the values then travel through that XCD's L2
+// with ordinary stores (device-scope write-through stores of this volume measured
+// 50 GB/s).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -51,13 +52,6 @@ __device__ __forceinline__ void dma16(const unsigned char *g, unsigned char *lds
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(l) : "memory", "m0");
 }
 
-// 16 bytes per lane written through to device memory (device-scope store): visible to every XCD once the
-// store is acknowledged, without a write-back of the whole L2.
-__device__ __forceinline__ void store16_device(v4f v, unsigned char *g)
-{
-    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(g), "v"(v) : "memory");
-}
-
 // The same with the LDS destination given as a byte address that is already wave-uniform (built from scalars).
 __device__ __forceinline__ void dma16_at(const unsigned char *g, uint32_t ldsAddr)
 {
@@ -80,12 +74,10 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 // Geometries (every wave computes 64 x 128: MB = 2 row blocks of 32, 4 column blocks of 32; two wave columns):
 //   WM 2 -> 128x256 tile, 4 waves, 3 stages (72 KiB LDS, two workgroups per CU);
 //   WM 4 -> 256x256 tile, 8 waves (128 KiB LDS, one workgroup per CU): half the L2 -> LDS traffic per MAC.
-//           PRESUM (WM 4 only) adds the 32 KiB ring of the peer pre-sum.
-template <uint32_t DT, int WM, bool PRESUM>
+template <uint32_t DT, int WM>
 __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
 {
     static_assert(WM == 2 || WM == 4, "supported geometries");
-    static_assert(!PRESUM || (WM == 4 && DT == DT_I8), "the pre-sum rides on the 256x256 W8A8 pipeline");
     using Acc = typename AccOf<DT>::type;
     constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
     constexpr int MB = 2;
@@ -100,11 +92,8 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     // One LDS pool, carved by constant offsets:
     //   BM = 128: three A stages (8 KiB each), then three B stages (16 KiB each)            = 72 KiB
     //   BM = 256: two A pair buffers (32 KiB each), then four B stages (16 KiB each)         = 128 KiB
-    //             PRESUM: then four ring slots of one KiB per wave                           = +32 KiB
     constexpr int POOL = (BM == 256) ? (4 * A_STAGE + 4 * B_STAGE) : 3 * (A_STAGE + B_STAGE);
-    constexpr int RING_SLOT = NW * 1024;
-    constexpr int LDS_BYTES = POOL + (PRESUM ? 4 * RING_SLOT : 0);
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[POOL];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -114,9 +103,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 
     const SchedParams &sp = args.sched;
     const bool linear = (args.flags & GF_LINEAR_ORDER) != 0;
-    const bool presum = PRESUM && args.presum != nullptr;
-    const uint32_t seq = launch_seq(sp, blockIdx.x, linear);
-    const uint32_t task = launch_task(sp, blockIdx.x, linear, args.keptRank, presum);
+    const uint32_t task = launch_task(sp, blockIdx.x, linear, args.keptRank);
     TileInfo ti;
     if (!task_tile(sp, task, ti)) return;
     // The kept tiles are the longest chain of a reduce-scatter launch (main loop, then the peers' partials):
@@ -225,8 +212,8 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     };
 
     // One k step, hand-scheduled: the 16 MFMAs of a wave are issued back to back, and every other
-    // instruction of the step (fragment reads for the NEXT eight MFMAs, the copies for later steps, the
-    // peer pre-sum) sits between two MFMAs, where it issues while the matrix pipe is busy.  The first
+    // instruction of the step (fragment reads for the NEXT eight MFMAs, the copies for later steps)
+    // sits between two MFMAs, where it issues while the matrix pipe is busy.  The first
     // eight MFMAs finish the previous step (fragments fa1/fb1, read during the previous step), the second
     // eight use fa0/fb0 read during the first eight; the MFMAs lag the fragment reads by half a step, so
     // LDS latency is never exposed.  The fences keep the compiler from regrouping the sequence.
@@ -348,18 +335,15 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         // The MFMAs lag the fragment reads by half a step: after the barrier of step kt the fragments of
         // (kt, kk=0) are read while the MFMAs of (kt-1, kk=1) run, so LDS latency is never exposed and a
         // stage only has to have landed at its own barrier.
-        // Copies a wave issues in step kt, in this order: B(kt+3) [B_DMA], on even kt the A pair (kt+2)/2
-        // [APC], and with PRESUM one 1 KiB piece of a peer's partial [PS].  The vector-memory counter retires
-        // in order, so "at most n outstanding" at the barrier of step s means everything older than the
-        // last n copies has landed:
-        //   even s needs A pair s/2 (issued in step s-2): younger are PS of step s-2 and all of step s-1;
+        // Copies a wave issues in step kt, in this order: B(kt+3) [B_DMA], then on even kt the A pair (kt+2)/2
+        // [APC].  The vector-memory counter retires in order, so "at most n outstanding" at the barrier of step
+        // s means everything older than the last n copies has landed:
+        //   even s needs A pair s/2 (issued in step s-2): younger are the copies of step s-1;
         //   odd s needs B(s) (issued in step s-3): younger are all of steps s-2 and s-1.
-        // Either way every copy of step s-3, the peer piece included, has landed at the barrier of step s.
         constexpr int AP = 256 * 128;   // bytes of an A pair buffer
         constexpr int APC = 32 / NW;    // pair copies per wave
-        constexpr int PS = PRESUM ? 1 : 0;
-        constexpr int WAIT_EVEN = PS + (B_DMA + PS);
-        constexpr int WAIT_ODD = (B_DMA + PS) + (B_DMA + APC + PS);
+        constexpr int WAIT_EVEN = B_DMA;
+        constexpr int WAIT_ODD = B_DMA + (B_DMA + APC);
         auto stAP = [&](uint32_t q) { return smem + (q & 1) * AP; };
         auto stB = [&](uint32_t step) { return smem + 2 * AP + (step & 3) * B_STAGE; };
         // pair copy j covers rows 8j..8j+7: lane -> row 8j + lane/8, slot lane&7 holds chunk slot ^ ((row>>1)&7)
@@ -385,55 +369,6 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             for (int mb = 0; mb < MB; ++mb) af[mb] = *(const v4i *)(sa + mb * 32 * 128);
         };
 
-        // ---- peer pre-sum state (PRESUM only) --------------------------------------------------------
-        // The scratch S is cut into units of NW KiB (one KiB per wave, within one row of S because n is a
-        // multiple of 256).  Producer i of nProd takes units i, i+nProd, ...; for each unit it copies the
-        // piece of peer 0, 1, ... in consecutive k steps, adds them in that order and stores the sum.
-        // Ring slot of the piece copied in step c is c & 3; it is added in step c + 3.
-        const uint32_t nP = args.nPeers;
-        const uint32_t nProd = args.presumProducers, nUnits = args.presumUnits;
-        const bool producer = presum && seq < nProd;
-        unsigned char *const ring = smem + POOL + w * 1024;
-        const uint32_t npr = args.N >> 8;   // KiB pieces per row of S
-        uint32_t iu = seq, ip = 0, cu = seq, cp = 0;
-        bool iact = producer && iu < nUnits, cact = iact;
-        auto unit_src = [&](uint32_t u) -> size_t {   // byte offset of this wave's piece of unit u in a peer buffer
-            const uint32_t g = u * NW + w, row = g / npr, cb = g - row * npr;
-            return ((size_t)(args.peerRowOffset + row) * args.peerLd + cb * 256) * 4 + lane * 16;
-        };
-        size_t ioff = iact ? unit_src(iu) : 0;
-        v4f psum = {0.f, 0.f, 0.f, 0.f};
-        auto peer_issue = [&](uint32_t slot) {
-            // always one copy, so the counts above hold; with nothing left to stream it re-reads cached A bytes
-            const unsigned char *src = Ag + lane * 16;
-            if (iact) {
-                src = (const unsigned char *)args.peers[ip] + ioff;
-                if (++ip == nP) {
-                    ip = 0;
-                    iu += nProd;
-                    iact = iu < nUnits;
-                    if (iact) ioff = unit_src(iu);
-                }
-            }
-            dma16_stream(src, ring + slot * RING_SLOT);
-        };
-        auto peer_read = [&](uint32_t slot) { return *(const v4f *)(ring + slot * RING_SLOT + lane * 16); };
-        auto peer_add = [&](v4f v) {
-            if (cp == 0) psum = v;
-            else {
-                psum.x = __fadd_rn(psum.x, v.x);
-                psum.y = __fadd_rn(psum.y, v.y);
-                psum.z = __fadd_rn(psum.z, v.z);
-                psum.w = __fadd_rn(psum.w, v.w);
-            }
-            if (++cp == nP) {
-                store16_device(psum, (unsigned char *)args.presum + ((size_t)cu * NW + w) * 1024 + lane * 16);
-                cp = 0;
-                cu += nProd;
-                cact = cu < nUnits;
-            }
-        };
-
         auto issue_step_b = [&](uint32_t kt, bool guard) {
             if (!guard || kt + 3 < nk) issue_b(offB4(kt + 3));
         };
@@ -451,7 +386,6 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         barrier_keep_vmem();
         issue_step_b(0, true);
         issue_step_a(0, true);
-        if constexpr (PRESUM) peer_issue(0);
         load_ap(fa0, 0, 0);
         load_b(fb0, stB(0), 0);
         load_ap(fa1, 0, 1);
@@ -461,29 +395,15 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         CATCOC_FENCE();
 
         auto compute = [&](uint32_t kt, bool guard) {
-            v4f pv;
-            bool padd = false;
             // The two waves that share a SIMD (w and w + 4) issue their copies in different halves of the step,
             // so that one of them always has MFMAs to feed the matrix pipe while the other computes addresses.
-            // (With the pre-sum every wave keeps the order B, A pair, peer piece that the wait counts assume.)
-            const bool early = PRESUM || ws < NW / 2;
+            const bool early = ws < NW / 2;
             sched_step([&](v4i (&af)[MB], int kk) { load_ap(af, kt, kk); }, stB(kt),
-                       [&] { if (early) issue_step_b(kt, guard); }, [&] { if (early) issue_step_a(kt, guard); },
+                       [&] { if (early) issue_step_b(kt, guard); }, [&] { if (early) issue_step_a(kt, guard); }, nothing,
                        [&] {
-                           if constexpr (PRESUM) {
-                               peer_issue(kt & 3);
-                               padd = cact && kt >= 3;
-                               if (padd) pv = peer_read((kt - 3) & 3);
-                           }
-                       },
-                       [&] {
-                           if constexpr (PRESUM) {
-                               if (padd) peer_add(pv);
-                           } else {
-                               if (!early) {
-                                   issue_step_b(kt, guard);
-                                   issue_step_a(kt, guard);
-                               }
+                           if (!early) {
+                               issue_step_b(kt, guard);
+                               issue_step_a(kt, guard);
                            }
                        });
         };
@@ -502,30 +422,6 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             compute(kt, true);
         }
         mma(fa1, fb1);
-
-        if constexpr (PRESUM) {
-            if (presum) {
-                // pieces copied in the last three steps, then whatever the main loop was too short for
-                CATCOC_WAIT_VMCNT(0);
-                for (uint32_t c = nk >= 3 ? nk - 3 : 0; c < nk; ++c)
-                    if (cact) peer_add(peer_read(c & 3));
-                while (cact) {
-                    uint32_t n = 0;
-                    while (n < 4 && iact) peer_issue(n++);
-                    CATCOC_WAIT_VMCNT(0);
-                    for (uint32_t i = 0; i < n; ++i) peer_add(peer_read(i));
-                    if (n == 0) break;   // cannot happen: the two sides walk the same sequence
-                }
-                if (seq < nProd) {
-                    // make this workgroup's part of S visible to the device, then count it
-                    // S was written through to memory (device-scope stores); once they are acknowledged
-                    // the count may go up, no cache-wide write-back needed
-                    CATCOC_WAIT_VMCNT(0);
-                    __syncthreads();
-                    if (tid == 0) __hip_atomic_fetch_add(args.presumCtl, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-            }
-        }
     }
 
 #undef CATCOC_FENCE
@@ -635,8 +531,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         }
 
         // one fp32 partial of the tile, added from global memory 32 rows (64 loads per lane) at a time
-        // (device: the partial was written by other workgroups of this launch, read it at device scope)
-        auto add_partial = [&](const float *base, int64_t ld, auto device) {
+        auto add_partial = [&](const float *base, int64_t ld) {
             const float *src = base + (size_t)row_base * ld + gcol0;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
@@ -644,11 +539,8 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
 #pragma unroll
-                    for (int nb = 0; nb < 4; ++nb) {
-                        const float *q = src + (size_t)(mb * 32 + (r >> 2) * 8 + (r & 3)) * ld + 32 * nb;
-                        if constexpr (decltype(device)::value) pv[r][nb] = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        else pv[r][nb] = __builtin_nontemporal_load(q);
-                    }
+                    for (int nb = 0; nb < 4; ++nb)
+                        pv[r][nb] = __builtin_nontemporal_load(src + (size_t)(mb * 32 + (r >> 2) * 8 + (r & 3)) * ld + 32 * nb);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
@@ -657,37 +549,8 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
-        const uint32_t nPeers = args.nPeers;
-        if (nPeers != 0) {
-            bool summed = false;
-            if constexpr (PRESUM) {
-                if (presum) {
-                    // wait (bounded) until every producer has counted its part of S
-                    volatile uint32_t *flag = (volatile uint32_t *)smem;
-                    __syncthreads();   // all waves are done with the LDS pool
-                    if (tid == 0) {
-                        uint32_t ok = 0;
-                        for (uint32_t i = 0; i < args.presumSpin; ++i) {
-                            if (__hip_atomic_load(args.presumCtl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= args.presumProducers) {
-                                ok = 1;
-                                break;
-                            }
-                            __builtin_amdgcn_s_sleep(32);
-                        }
-                        *flag = ok;
-                    }
-                    __syncthreads();
-                    summed = *flag != 0;
-
-                }
-            }
-            if (summed) {
-                add_partial(args.presum + (size_t)out_row0 * args.N, args.N, std::true_type{});
-            } else {
-                for (uint32_t p = 0; p < nPeers; ++p)
-                    add_partial((const float *)args.peers[p] + (size_t)(args.peerRowOffset + out_row0) * args.peerLd, args.peerLd, std::false_type{});
-            }
-        }
+        for (uint32_t p = 0; p < args.nPeers; ++p)
+            add_partial((const float *)args.peers[p] + (size_t)(args.peerRowOffset + out_row0) * args.peerLd, args.peerLd);
 
         // 16-bit output.  A lane holds single columns 32 apart, so storing from registers would write 64-byte
         // pieces (half a cache line each, 128 store instructions per lane).  Instead every wave turns its 64 x 128
@@ -763,17 +626,6 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         }
     }
 
-    if constexpr (PRESUM) {
-        // the last workgroup of the launch to get here re-arms the counters for the next launch: by then
-        // every producer has counted itself and every kept tile has stopped looking at the count
-        if (presum && tid == 0) {
-            const uint32_t fin = __hip_atomic_fetch_add(args.presumCtl + 1, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-            if (fin + 1 == sp.coreLoops) {
-                __hip_atomic_store(args.presumCtl, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(args.presumCtl + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-    }
 }
 
 }  // namespace catcoc

@@ -13,9 +13,9 @@ int launch_gemm_dma_f16(const GemmArgs &args, void *stream)
 {
     const dim3 grid(args.sched.coreLoops);
     if (args.sched.m0 == 256)
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_F16, 4, false>), grid, dim3(512), 0, (hipStream_t)stream, args);
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_F16, 4>), grid, dim3(512), 0, (hipStream_t)stream, args);
     else
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_F16, 2, false>), grid, dim3(256), 0, (hipStream_t)stream, args);
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_F16, 2>), grid, dim3(256), 0, (hipStream_t)stream, args);
     return (int)hipGetLastError();
 }
 }  // namespace catcoc

@@ -9,16 +9,14 @@ int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream)
 }
 
 // Full-tile paths with direct-to-LDS copies (see gemm_dma_kernel.h for their requirements):
-// m0 = 128 (4 waves) or m0 = 256 (8 waves, optionally with the peer pre-sum).
+// m0 = 128 (4 waves, two workgroups per CU) or m0 = 256 (8 waves).
 int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
 {
     const dim3 grid(args.sched.coreLoops);
-    if (args.sched.m0 == 256 && args.presum != nullptr)
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, true>), grid, dim3(512), 0, (hipStream_t)stream, args);
-    else if (args.sched.m0 == 256)
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, false>), grid, dim3(512), 0, (hipStream_t)stream, args);
+    if (args.sched.m0 == 256)
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), grid, dim3(512), 0, (hipStream_t)stream, args);
     else
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false>), grid, dim3(256), 0, (hipStream_t)stream, args);
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2>), grid, dim3(256), 0, (hipStream_t)stream, args);
     return (int)hipGetLastError();
 }
 }  // namespace catcoc

@@ -251,19 +251,6 @@ CATCOC_HD uint32_t kept_first_task(const SchedParams &s, uint32_t keptRank, uint
     return round * bpc + b;
 }
 
-// The same with the kept tasks LAST (used when the other workgroups prepare the kept tiles' peer sum,
-// which has to be complete before a kept tile can finish).  A bijection.
-CATCOC_HD uint32_t kept_order_task(const SchedParams &s, uint32_t keptRank, uint32_t seq, bool keptLast)
-{
-    if (!keptLast || s.op != OP_REDUCE_SCATTER || s.P <= 1) return kept_first_task(s, keptRank, seq);
-    const uint32_t keptCount = s.coreLoops / s.P;
-    const uint32_t others = s.coreLoops - keptCount;
-    return kept_first_task(s, keptRank, seq < others ? seq + keptCount : seq - others);
-}
-
-// Position of a workgroup in the launch sequence (XCD-aware chunking).
-CATCOC_HD uint32_t launch_seq(const SchedParams &s, uint32_t wg, bool linear) { return workgroup_task(wg, s.coreLoops, linear); }
-
 // XCD-block launch order for reduce-scatter and all-reduce launches.  Consecutive workgroups go round-robin to the
 // 8 XCDs, each with its own L2, so XCD x = wg mod 8 is given one block of the global tile grid (all ranks' rows):
 // the grid is cut RX x CX = 8 ways, rows dealt round-robin to the RX row parts (every part then holds the same share
@@ -271,9 +258,17 @@ CATCOC_HD uint32_t launch_seq(const SchedParams &s, uint32_t wg, bool linear) { 
 // the A rows plus B columns one XCD touches.  Inside its block an XCD walks row by row with the kept rank's rows
 // first, so the tiles in flight on an XCD at any time share a few A row blocks and all of the block's B columns.
 // Returns false when the grid does not divide evenly (callers fall back to the chunked order).
-CATCOC_HD bool xcd_block_task(const SchedParams &s, uint32_t keptRank, uint32_t wg, uint32_t &task)
+struct XcdBlock {
+    uint32_t RX, CX;          // row parts x column parts = 8
+    uint32_t rowsPer, colsPer;  // tile rows / tile columns of one XCD's block
+    uint32_t rp, cp;          // this XCD's row part and column part
+    uint32_t i0, i1;          // the block's tile rows rp + RX*i with i in [i0, i1) belong to the kept rank
+};
+
+// Geometry of XCD x's block; false when the order does not apply to this launch.
+CATCOC_HD bool xcd_block(const SchedParams &s, uint32_t keptRank, uint32_t x, XcdBlock &g)
 {
-    if (s.op == OP_ALLGATHER || (s.coreLoops & 7u) != 0 || wg >= s.coreLoops) return false;
+    if (s.op == OP_ALLGATHER || (s.coreLoops & 7u) != 0) return false;
     const bool rs = s.op == OP_REDUCE_SCATTER;
     const uint32_t GM = (rs ? s.P : 1u) * s.loopsM;
     if (GM * s.loopsN != s.coreLoops) return false;
@@ -285,27 +280,35 @@ CATCOC_HD bool xcd_block_task(const SchedParams &s, uint32_t keptRank, uint32_t 
         if (cost < best) { best = cost; RX = r; }
     }
     if (RX == 0) return false;
-    const uint32_t CX = 8u / RX, rowsPer = GM / RX, colsPer = s.loopsN / CX;
-    const uint32_t x = wg & 7u, j = wg >> 3;
-    const uint32_t rp = x / CX, cp = x - rp * CX;
-    const uint32_t ri = j / colsPer, ci = j - ri * colsPer;
-    // rows of this part are rp + RX*i; those of the kept rank are i in [i0, i1)
-    uint32_t i0 = 0, i1 = 0;
+    g.RX = RX;
+    g.CX = 8u / RX;
+    g.rowsPer = GM / RX;
+    g.colsPer = s.loopsN / g.CX;
+    g.rp = x / g.CX;
+    g.cp = x - g.rp * g.CX;
+    g.i0 = g.i1 = 0;
     if (rs && s.P > 1) {
         const uint32_t lo = keptRank * s.loopsM, hi = lo + s.loopsM;
-        i0 = lo > rp ? ceil_div(lo - rp, RX) : 0u;
-        i1 = hi > rp ? ceil_div(hi - rp, RX) : 0u;
-        i0 = umin(i0, rowsPer);
-        i1 = umin(i1, rowsPer);
+        g.i0 = umin(lo > g.rp ? ceil_div(lo - g.rp, RX) : 0u, g.rowsPer);
+        g.i1 = umin(hi > g.rp ? ceil_div(hi - g.rp, RX) : 0u, g.rowsPer);
     }
-    const uint32_t nk = i1 - i0;
+    return true;
+}
+
+CATCOC_HD bool xcd_block_task(const SchedParams &s, uint32_t keptRank, uint32_t wg, uint32_t &task)
+{
+    XcdBlock g;
+    if (wg >= s.coreLoops || !xcd_block(s, keptRank, wg & 7u, g)) return false;
+    const uint32_t j = wg >> 3;
+    const uint32_t ri = j / g.colsPer, ci = j - ri * g.colsPer;
+    const uint32_t nk = g.i1 - g.i0;
     uint32_t i;
-    if (ri < nk) i = i0 + ri;
-    else { const uint32_t t = ri - nk; i = t < i0 ? t : t + nk; }
-    const uint32_t gr = rp + RX * i, nIdx = cp * colsPer + ci;
+    if (ri < nk) i = g.i0 + ri;
+    else { const uint32_t t = ri - nk; i = t < g.i0 ? t : t + nk; }
+    const uint32_t gr = g.rp + g.RX * i, nIdx = g.cp * g.colsPer + ci;
     const uint32_t rank = gr / s.loopsM, mIdx = gr - rank * s.loopsM;
     const uint32_t inRank = swizzle_block_index(s.off, s.dir, s.loopsM, s.loopsN, mIdx, nIdx);
-    if (!rs) { task = inRank; return true; }
+    if (s.op != OP_REDUCE_SCATTER) { task = inRank; return true; }
     const uint32_t perRank = s.blockPerComm / s.P;
     const uint32_t round = inRank / perRank, idx = inRank - round * perRank;
     const uint32_t commLoops = ceil_div(s.coreLoops, s.blockPerComm);
@@ -315,13 +318,13 @@ CATCOC_HD bool xcd_block_task(const SchedParams &s, uint32_t keptRank, uint32_t 
 }
 
 // Workgroup -> task of a launch: the XCD-block order where it applies, else XCD-aware chunking with the kept
-// rank's tiles first (last when the other tiles pre-sum the peers for them).
-CATCOC_HD uint32_t launch_task(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank, bool keptLast)
+// rank's tiles first.  Either way the kept tiles are among the first ceil(kept / 128) * 128 workgroups.
+CATCOC_HD uint32_t launch_task(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank)
 {
     if (linear) return wg;
     uint32_t task;
-    if (!keptLast && xcd_block_task(s, keptRank, wg, task)) return task;
-    return kept_order_task(s, keptRank, workgroup_task(wg, s.coreLoops, false), keptLast);
+    if (xcd_block_task(s, keptRank, wg, task)) return task;
+    return kept_first_task(s, keptRank, workgroup_task(wg, s.coreLoops, false));
 }
 
 // Workgroup -> task of a launch: XCD-aware chunking, then kept-first ordering.

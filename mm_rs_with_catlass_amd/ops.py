@@ -59,7 +59,7 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
                                         out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
                                         reduce_int32=False, outbound=None, checksum=None, acc_dump=None,
                                         c_accum=None, block_num=0, stages=0, swizzle=None, linear_order=False,
-                                        out=None, workspace=None, wait_polls=0):
+                                        out=None):
     """Validate and bind the arguments once; returns (launch, out) where launch() enqueues one call of
     catcoc_launch_quant_matmul_reduce_scatter on torch's current stream (for launch-rate-sensitive loops)."""
     _check_dev(x1, x2, scale_x1, scale_x2, bias, outbound, checksum, acc_dump, c_accum, *peers)
@@ -69,15 +69,10 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
     flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_REDUCE_INT32 if reduce_int32 else 0) | \
         (_l.FLAG_LINEAR_ORDER if linear_order else 0)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
-    if workspace is not None:
-        _check_dev(workspace)
-        d.workspace = workspace.data_ptr()
-        d.workspaceBytes = workspace.numel() * workspace.element_size()
-        d.reduceWaitPolls = wait_polls
     if out is None:
         out = torch.empty((m // max(rank_size, 1), n), dtype=out_dtype, device=x1.device)
     L = _l.load()
-    keep = (x1, x2, scale_x1, scale_x2, bias, tuple(peers), outbound, checksum, acc_dump, c_accum, out, d, t, workspace)
+    keep = (x1, x2, scale_x1, scale_x2, bias, tuple(peers), outbound, checksum, acc_dump, c_accum, out, d, t)
     fn = L.catcoc_launch_quant_matmul_reduce_scatter
     argv = (0, x1.data_ptr(), x2.data_ptr(), scale_x1.data_ptr(), scale_x2.data_ptr(), _ptr(bias), _ptr(c_accum),
             out.data_ptr(), C.addressof(d), C.byref(t), 0, int(trans_b), _TORCH_TO_DT[out.dtype])
@@ -91,20 +86,17 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
 def quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(), rank=0, rank_size=1,
                                 out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
                                 reduce_int32=False, outbound=None, checksum=None, acc_dump=None, c_accum=None,
-                                block_num=0, stages=0, swizzle=None, linear_order=False, out=None, workspace=None,
-                                wait_polls=0):
+                                block_num=0, stages=0, swizzle=None, linear_order=False, out=None):
     """W8A8 matmul -> reduce-scatter share of one rank.
 
     x1 [m,k] int8, x2 [k,n] int8 ([n,k] with trans_b), scale_x1 [m] fp32 per token, scale_x2 [n] fp32 per
     channel, bias [n] int32 or None.  peers: rank_size-1 staged partials for the kept rows (fp32, or int32
-    with reduce_int32), added in list order after the local partial.  workspace: optional zero-initialised
-    uint8 tensor of reduce_workspace_size() bytes that lets the other ranks' tiles pre-sum the peers.
+    with reduce_int32), added in list order after the local partial.
     Returns d_out [m/rank_size, n].
     """
     launch, out = prepare_quant_matmul_reduce_scatter(
         x1, x2, scale_x1, scale_x2, bias, peers, rank, rank_size, out_dtype, tiling, trans_b, peer_row_offset,
-        reduce_int32, outbound, checksum, acc_dump, c_accum, block_num, stages, swizzle, linear_order, out, workspace,
-        wait_polls)
+        reduce_int32, outbound, checksum, acc_dump, c_accum, block_num, stages, swizzle, linear_order, out)
     launch()
     _l.check()
     return out
@@ -156,13 +148,6 @@ def quant_matmul_splitk(*args, **kw):
     launch()
     _l.check()
     return out
-
-
-def reduce_workspace_size(m, k, n, rank, rank_size, tiling=None):
-    """Bytes of the optional pre-sum workspace of quant_matmul_reduce_scatter (0 = this shape cannot use one)."""
-    t = tiling if tiling is not None else default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
-    d = _l.make_desc(rank, rank_size)
-    return int(_l.load().catcoc_get_reduce_workspace_size(C.byref(t), C.byref(d)))
 
 
 def _float_op(comm_type, a, b, c_shape, peers, rank, rank_size, tiling, trans_a, trans_b, peer_row_offset, outbound,

@@ -143,19 +143,14 @@ def test_launch_order_is_a_bijection_with_kept_tiles_first_or_last(so):
                 kept.append(tr.value == rank)
             nk = sum(kept)
             assert nk == n // P
-            presum = ws and m0 == 256          # the pre-sum rides on 256-row tiles only
-            # the kept tiles are the first workgroups to be dispatched (the last ones with a pre-sum workspace),
-            # up to the permutation inside a block of 128 workgroups that the XCD-aware orders apply
+            # the kept tiles are the first workgroups to be dispatched, up to the permutation inside a block of
+            # 128 workgroups that the XCD-aware orders apply
             span = -(-nk // 128) * 128
-            wgs = [wg for wg in range(n) if kept[wg]]
-            assert (min(wgs) >= n - span) if presum else (max(wgs) < span)
+            assert max(wg for wg in range(n) if kept[wg]) < span
 
 
 def test_workspace_size_queries(so):
     from mm_rs_with_catlass_amd import ops
-    assert ops.reduce_workspace_size(8192, 1792, 4096, 0, 8) == 1024 * 4096 * 4 + 256
-    assert ops.reduce_workspace_size(8192, 1792 + 64, 4096, 0, 8) == 0          # k not a multiple of 128
-    assert ops.reduce_workspace_size(8192 + 8, 1792, 4096, 0, 8) == 0           # ragged rows
     need, f, tiles = ops.splitk_plan(16, 8192, 8192, 8, 0, 2)
     assert (f, tiles) == (oracle.splitk_factor(16, 8192, 8192, 256, 128, 128, 256), 64)
     assert need == f * tiles * 128 * 128 * 4 + 256
