@@ -86,6 +86,74 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         }
     };
 
+    // ---- everything the epilogue reads is requested now, before the stream starts ---------------
+    // The tail of this kernel is a chain of memory round trips (publish, count, fetch the other slices); bias,
+    // scales and the peers' values of the tile's first 32-row block with kept rows would add two more, so every
+    // slice asks for them here and holds them in registers (the peers of a decode tile are a few KiB).  A wave
+    // can have 63 memory operations outstanding and this code runs once, so it is kept short: one load per
+    // 32-row block for the per-token scales (lane l fetches row l of the block; the lanes pick their rows from
+    // each other in the epilogue), and peer loads only for the register slots whose rows can be kept rows.
+    //
+    // acc[mb][r] is element (lrow, lcol) with lrow = mb*32 + slot_row(r) + 4h, lcol = w*32 + c32.  Inside block mb
+    // the kept rows are the local rows [kLo, kHi) (wave-uniform); lane and slot then decide with one unsigned
+    // compare, (slot_row(r) + rel) < kHi - kLo with rel = 4h - kLo, and a peer offset is base + slot_row(r) * pitch.
+    const uint32_t lcol = w * 32 + c32;
+    const uint32_t gcol = colT + lcol;
+    const uint32_t keptEnd = args.keptBegin + args.keptRows;
+    const uint64_t peerBytes = (uint64_t)(args.peerRowOffset + args.keptRows) * args.peerLd * 4;
+    const int peerRange = peerBytes > 0x7fffffffull ? 0x7fffffff : (int)peerBytes;
+    const uint32_t peerPitch = (uint32_t)args.peerLd * 4u;
+    constexpr uint32_t OUT_OF_RANGE = 0x7fffffffu;   // a buffer load at this offset touches no memory and reads zero
+    auto slot_row = [](int r) { return (uint32_t)((r >> 2) * 8 + (r & 3)); };
+    struct KeptRows { uint32_t lo, n, rel, base; };   // of one 32-row block
+    auto kept_rows = [&](uint32_t mb) {
+        const uint32_t blk0 = row0 + mb * 32, blkEnd = row0 + umin(rowsValid, mb * 32 + 32);
+        const uint32_t lo = args.keptBegin > blk0 ? args.keptBegin : blk0, hi = umin(keptEnd, blkEnd);
+        KeptRows k;
+        k.lo = lo - blk0;
+        k.n = hi > lo ? hi - lo : 0u;
+        k.rel = 4u * h - k.lo;
+        k.base = ((uint32_t)(args.peerRowOffset + blk0 - args.keptBegin) + 4u * h) * peerPitch + gcol * 4u;
+        return k;
+    };
+    auto slot_active = [&](const KeptRows &k, int r) { return slot_row(r) < k.lo + k.n && slot_row(r) + 4u >= k.lo; };   // uniform
+    auto lane_kept = [&](const KeptRows &k, int r) { return slot_row(r) + k.rel < k.n; };
+    // eight peers of one block, slot by slot: one uniform test, then eight loads back to back
+    auto fetch_peers = [&](const KeptRows &k, uint32_t p0, float (&pv)[8][16]) {
+        __amdgpu_buffer_rsrc_t prs[8];   // a peer that does not exist gets an empty range
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const bool use = p0 + q < args.nPeers && k.n != 0;
+            prs[q] = __builtin_amdgcn_make_buffer_rsrc((void *)args.peers[use ? p0 + q : 0], 0, use ? peerRange : 0, 0x00020000);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            if (k.n != 0 && slot_active(k, r)) {
+                const uint32_t off = lane_kept(k, r) ? k.base + slot_row(r) * peerPitch : OUT_OF_RANGE;
+#pragma unroll
+                for (int q = 0; q < 8; ++q)
+                    pv[q][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(prs[q], off, 0, 2 /* streaming */));
+            } else {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) pv[q][r] = 0.0f;
+            }
+        }
+    };
+    uint32_t mbK = 0;   // first 32-row block of the tile with kept rows (none: block 0, which then has nothing to fetch)
+#pragma unroll
+    for (int mb = MBW - 1; mb >= 0; --mb)
+        if (kept_rows(mb).n != 0) mbK = mb;
+    const int bv = args.bias ? args.bias[gcol] : 0;
+    const float sN = args.scaleN[gcol];
+    float sMrow[MBW];   // nothing fetched here is looked at before the stream has run
+#pragma unroll
+    for (int mb = 0; mb < MBW; ++mb) {
+        const uint32_t lrow = mb * 32 + c32;
+        sMrow[mb] = lrow < rowsValid ? args.scaleM[row0 + lrow] : 0.0f;
+    }
+    float pv0[8][16];
+    fetch_peers(kept_rows(mbK), 0, pv0);
+
     v16i acc[MBW];
 #pragma unroll
     for (int mb = 0; mb < MBW; ++mb)
@@ -137,23 +205,25 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     }
 
     // ---- k slices meet -------------------------------------------------------------
-    // acc[mb][r] is element (lrow, lcol) with lrow = mb*32 + (r>>2)*8 + h*4 + (r&3), lcol = w*32 + c32
-    const uint32_t lcol = w * 32 + c32;
     if (f > 1) {
         // Partial tiles travel through memory at device scope (cache policy sc1: written through / read past
-        // the XCD-local L2), as ordinary buffer accesses so that the loads of a slice are issued together.
+        // the XCD-local L2), as ordinary buffer accesses so that the loads of a slice are issued together.  Inside
+        // the workspace a tile is kept in register order: int32 index ((mb*4 + g)*256 + thread)*4 + j holds register
+        // r = 4g + j of block mb, so every access is 16 bytes per lane and 1 KiB per wave.  Groups of rows past the
+        // end of A are neither written nor read.
         constexpr int DEVICE_SCOPE = 16;   // sc1
         const size_t tileBytes = 128 * 128 * 4;
+        auto group_valid = [&](int mb, int g) { return (uint32_t)(mb * 32 + g * 8) < rowsValid; };   // wave-uniform
         const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
             (void *)(args.skPart + ((size_t)slice * loopsM * loopsN + tile) * (128 * 128)), 0, (int)tileBytes, 0x00020000);
 #pragma unroll
         for (int mb = 0; mb < MBW; ++mb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint32_t lrow = mb * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
-                const int iv = acc[mb][r];
-                if (lrow < rowsValid) __builtin_amdgcn_raw_buffer_store_b32(iv, mine, (lrow * 128 + lcol) * 4, 0, DEVICE_SCOPE);
-            }
+            for (int g = 0; g < 4; ++g)
+                if (group_valid(mb, g)) {
+                    const v4i iv = {acc[mb][4 * g], acc[mb][4 * g + 1], acc[mb][4 * g + 2], acc[mb][4 * g + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(iv, mine, ((mb * 4 + g) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+                }
         // once the stores are acknowledged the slice may be counted
         CATCOC_WAIT_VMCNT(0);
         __syncthreads();
@@ -162,89 +232,101 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         __syncthreads();
         if (*flag != f - 1u) return;
         if (tid == 0) __hip_atomic_store(args.skCount + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // the other slices' partials, one 32-row block at a time and up to four slices per round trip
+        // the other slices' partials: every 32-row block of up to three slices per round trip
         const int32_t *tile0 = args.skPart + (size_t)tile * (128 * 128);
         const size_t sliceStride = (size_t)loopsM * loopsN * (128 * 128);
+        constexpr int QG = 3;
+        for (uint32_t o0 = 0; o0 + 1 < f; o0 += QG) {
+            v4i pv[QG][MBW][4];
 #pragma unroll
-        for (int mb = 0; mb < MBW; ++mb) {
-            for (uint32_t s0 = 0; s0 < f; s0 += 4) {
-                int pv[4][16];
+            for (int q = 0; q < QG; ++q) {
+                const uint32_t o = o0 + q;                       // o-th of the f - 1 other slices
+                const bool use = o + 1 < f;
+                const uint32_t sl = o < slice ? o : o + 1;
+                const __amdgpu_buffer_rsrc_t other = __builtin_amdgcn_make_buffer_rsrc(
+                    (void *)(tile0 + (use ? sl : slice) * sliceStride), 0, use ? (int)tileBytes : 0, 0x00020000);
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const uint32_t s = s0 + q;
-                    const bool use = s < f && s != slice;
-                    const __amdgpu_buffer_rsrc_t other = __builtin_amdgcn_make_buffer_rsrc(
-                        (void *)(tile0 + (use ? s : slice) * sliceStride), 0, (int)tileBytes, 0x00020000);
+                for (int mb = 0; mb < MBW; ++mb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const uint32_t lrow = mb * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
-                        // unused slots and rows past the end read as zero: the offset is pushed out of the descriptor's range
-                        pv[q][r] = __builtin_amdgcn_raw_buffer_load_b32(other, (use && lrow < rowsValid) ? (lrow * 128 + lcol) * 4 : 0x7fffffff, 0, DEVICE_SCOPE);
+                    for (int g = 0; g < 4; ++g) {
+                        pv[q][mb][g] = v4i{0, 0, 0, 0};
+                        if (use && group_valid(mb, g))
+                            pv[q][mb][g] = __builtin_amdgcn_raw_buffer_load_b128(other, ((mb * 4 + g) * 256 + tid) * 16, 0, DEVICE_SCOPE);
                     }
-                }
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[mb][r] += pv[q][r];
             }
+#pragma unroll
+            for (int q = 0; q < QG; ++q)
+#pragma unroll
+                for (int mb = 0; mb < MBW; ++mb)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        acc[mb][4 * g] += pv[q][mb][g].x;
+                        acc[mb][4 * g + 1] += pv[q][mb][g].y;
+                        acc[mb][4 * g + 2] += pv[q][mb][g].z;
+                        acc[mb][4 * g + 3] += pv[q][mb][g].w;
+                    }
         }
     }
 
     // ---- epilogue on the rows that exist -----------------------------------------------
-    // Per 32-row block: bias, dumps, dequant; then the peers' values of the block's kept rows are fetched eight
-    // peers at a time in ONE round trip (out-of-range offsets of a buffer load cost nothing and return zero, which
-    // masks rows that are not kept and peers that do not exist) and added in slot order; then the 16-bit store.
-    const uint32_t gcol = colT + lcol;
-    const int bv = args.bias ? args.bias[gcol] : 0;
-    const float sN = args.scaleN[gcol];
-    const uint32_t keptEnd = args.keptBegin + args.keptRows;
-    const uint64_t peerBytes = (uint64_t)(args.peerRowOffset + args.keptRows) * args.peerLd * 4;
-    const int peerRange = peerBytes > 0x7fffffffull ? 0x7fffffff : (int)peerBytes;
+    // Per 32-row block: bias, dumps, checksum of the rows that are not kept; then, for the register slots that
+    // hold kept rows only, dequant, the peers in slot order (the first block with kept rows has its first eight
+    // peers in registers already; anything else is fetched eight peers at a time in one round trip) and the
+    // 16-bit store.
     long long csum = 0;
 #pragma unroll
     for (int mb = 0; mb < MBW; ++mb) {
-        const uint32_t blk0 = row0 + mb * 32;
-        if (blk0 >= row0 + rowsValid) break;
-        float v[16];
-        uint32_t poff[16];
+        if ((uint32_t)mb * 32 >= rowsValid) break;
+        const KeptRows k = kept_rows(mb);
+        const uint32_t vrel = mb * 32 + 4u * h;   // slot r is a row of A when slot_row(r) + vrel < rowsValid
+        int iv[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const uint32_t lrow = mb * 32 + (r >> 2) * 8 + h * 4 + (r & 3);
-            const uint32_t grow = row0 + lrow;
-            const bool valid = lrow < rowsValid;
-            const bool kept = valid && grow >= args.keptBegin && grow < keptEnd;
-            const int iv = acc[mb][r] + bv;
-            if (valid && args.accDump) ((int32_t *)args.accDump)[(size_t)grow * N + gcol] = iv;
-            if (kept && args.cAccum) args.cAccum[(size_t)(grow - args.keptBegin) * N + gcol] = iv;
-            if (valid && !kept) csum += iv;
-            v[r] = __fmul_rn(__fmul_rn((float)iv, sN), args.scaleM[valid ? grow : row0]);
-            poff[r] = kept ? (uint32_t)(((args.peerRowOffset + grow - args.keptBegin) * args.peerLd + gcol) * 4) : 0x7fffffffu;
+            iv[r] = acc[mb][r] + bv;
+            csum += (slot_row(r) + vrel < rowsValid && !lane_kept(k, r)) ? iv[r] : 0;
         }
-        if (blk0 < keptEnd && blk0 + 32 > args.keptBegin) {   // the block holds kept rows
-            for (uint32_t p0 = 0; p0 < args.nPeers; p0 += 8) {
-                float pv[8][16];
+        if (args.accDump) {
 #pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    const bool use = p0 + q < args.nPeers;
-                    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-                        (void *)args.peers[use ? p0 + q : 0], 0, use ? peerRange : 0, 0x00020000);
+            for (int r = 0; r < 16; ++r)
+                if (slot_row(r) + vrel < rowsValid) ((int32_t *)args.accDump)[(size_t)(row0 + vrel + slot_row(r)) * N + gcol] = iv[r];
+        }
+        if (k.n == 0) continue;
+        if (args.cAccum) {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        pv[q][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, poff[r], 0, 2 /* streaming */));
+            for (int r = 0; r < 16; ++r)
+                if (lane_kept(k, r)) args.cAccum[(size_t)(row0 + vrel + slot_row(r) - args.keptBegin) * N + gcol] = iv[r];
+        }
+        float v[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            v[r] = slot_active(k, r) ? __fmul_rn(__fmul_rn((float)iv[r], sN), __shfl(sMrow[mb], slot_row(r) + 4 * h, 64)) : 0.0f;
+        uint32_t p0 = 0;
+        if ((uint32_t)mb == mbK) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (slot_active(k, r)) {
+#pragma unroll
+                    for (int q = 0; q < 8; ++q)
+                        if ((uint32_t)q < args.nPeers) v[r] = __fadd_rn(v[r], pv0[q][r]);
                 }
-#pragma unroll
-                for (int q = 0; q < 8; ++q)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        if (p0 + q < args.nPeers) v[r] = __fadd_rn(v[r], pv[q][r]);
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint32_t grow = blk0 + (r >> 2) * 8 + h * 4 + (r & 3);
-                if (poff[r] != 0x7fffffffu)
-                    ((unsigned short *)args.d)[(size_t)(grow - args.keptBegin) * args.ldd + gcol] = (unsigned short)f32_to_out16(v[r], args.outDtype);
-            }
+            p0 = 8;
         }
+        for (; p0 < args.nPeers; p0 += 8) {
+            float pv[8][16];
+            fetch_peers(k, p0, pv);
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (slot_active(k, r)) {
+#pragma unroll
+                    for (int q = 0; q < 8; ++q)
+                        if (p0 + q < args.nPeers) v[r] = __fadd_rn(v[r], pv[q][r]);
+                }
+        }
+        // signed: the block may start above the first kept row (only kept lanes dereference)
+        unsigned short *drow = (unsigned short *)args.d + ((int64_t)(row0 + vrel) - (int64_t)args.keptBegin) * args.ldd + gcol;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            if (slot_active(k, r) && lane_kept(k, r)) drow[(int64_t)slot_row(r) * args.ldd] = (unsigned short)f32_to_out16(v[r], args.outDtype);
     }
     if (args.checksum != nullptr) {
         long long *red = (long long *)smem + 8;
