@@ -4,9 +4,9 @@
 // decode-sized problem still spreads over every CU with a small split factor.
 //
 // A workgroup (4 waves) streams its k slice of B (64 k rows x 128 columns = 8 KiB per
-// step) and of A straight into an 8-stage LDS ring with direct-to-LDS copies, seven
-// steps ahead, so about 100 KiB per CU is in flight; every wave multiplies all rows
-// of the tile by its own 32 columns.  Partial tiles of the k slices are written
+// step) and of A straight into an LDS ring of 8 or 12 stages with direct-to-LDS copies,
+// so 60 to 80 KiB per CU is in flight; every wave multiplies all rows of the tile by
+// its own 32 columns, two or four steps per barrier.  Partial tiles of the k slices are written
 // through to memory as int32 (device-scope stores), a per-tile counter elects the
 // last slice to arrive, and that workgroup adds the other partials (integer adds:
 // exact in any order), then runs the same epilogue as the large-M kernels on the
@@ -20,6 +20,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "gemm_dma_kernel.h"
 
 namespace catcoc {
@@ -30,7 +32,8 @@ template <int MBW>
 __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args)
 {
     constexpr int NW = 4;
-    constexpr int NS = 8;
+    constexpr int G = (MBW == 1) ? 4 : 2;      // k steps per barrier
+    constexpr int NS = (MBW == 1) ? 12 : 8;    // LDS stages (a multiple of G, at least 2G)
     constexpr int ROWS = 32 * MBW;
     constexpr int A_STAGE = ROWS * 64;
     constexpr int B_STAGE = 64 * 128;
@@ -86,13 +89,14 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         }
     };
 
-    // ---- everything the epilogue reads is requested now, before the stream starts ---------------
+    // ---- everything the epilogue reads is requested while the stream is still in flight ---------
     // The tail of this kernel is a chain of memory round trips (publish, count, fetch the other slices); bias,
     // scales and the peers' values of the tile's first 32-row block with kept rows would add two more, so every
-    // slice asks for them here and holds them in registers (the peers of a decode tile are a few KiB).  A wave
-    // can have 63 memory operations outstanding and this code runs once, so it is kept short: one load per
-    // 32-row block for the per-token scales (lane l fetches row l of the block; the lanes pick their rows from
-    // each other in the epilogue), and peer loads only for the register slots whose rows can be kept rows.
+    // slice asks for them as soon as its last copy of B is on its way (request_epilogue_operands below) and holds
+    // them in registers (the peers of a decode tile are a few KiB).  A wave can have 63 memory operations
+    // outstanding and this code runs once, so it is kept short: one load per 32-row block for the per-token
+    // scales (lane l fetches row l of the block; the lanes pick their rows from each other in the epilogue), and
+    // peer loads only for the register slots whose rows can be kept rows.
     //
     // acc[mb][r] is element (lrow, lcol) with lrow = mb*32 + slot_row(r) + 4h, lcol = w*32 + c32.  Inside block mb
     // the kept rows are the local rows [kLo, kHi) (wave-uniform); lane and slot then decide with one unsigned
@@ -143,16 +147,20 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
 #pragma unroll
     for (int mb = MBW - 1; mb >= 0; --mb)
         if (kept_rows(mb).n != 0) mbK = mb;
-    const int bv = args.bias ? args.bias[gcol] : 0;
-    const float sN = args.scaleN[gcol];
-    float sMrow[MBW];   // nothing fetched here is looked at before the stream has run
-#pragma unroll
-    for (int mb = 0; mb < MBW; ++mb) {
-        const uint32_t lrow = mb * 32 + c32;
-        sMrow[mb] = lrow < rowsValid ? args.scaleM[row0 + lrow] : 0.0f;
-    }
+    int bv;
+    float sN;
+    float sMrow[MBW];
     float pv0[8][16];
-    fetch_peers(kept_rows(mbK), 0, pv0);
+    auto request_epilogue_operands = [&]() {
+        bv = args.bias ? args.bias[gcol] : 0;
+        sN = args.scaleN[gcol];
+#pragma unroll
+        for (int mb = 0; mb < MBW; ++mb) {
+            const uint32_t lrow = mb * 32 + c32;
+            sMrow[mb] = lrow < rowsValid ? args.scaleM[row0 + lrow] : 0.0f;
+        }
+        fetch_peers(kept_rows(mbK), 0, pv0);
+    };
 
     v16i acc[MBW];
 #pragma unroll
@@ -166,43 +174,68 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     const int ti16 = lane & 15, tch = (lane >> 4) & 1, trow = ti16 >> 1, thalf = ti16 & 1;
     const uint32_t b_lds = (16 * h + trow) * 128 + (((2 * w + tch) ^ (((trow >> 1) & 3) << 1)) * 16) + thalf * 8;
 
-    const uint32_t pre = umin(nsteps, NS - 1);
-    for (uint32_t i = 0; i < pre; ++i) issue(i, i);
-    for (uint32_t kt = 0; kt < nsteps; ++kt) {
-        const uint32_t ahead = umin(nsteps - 1u - kt, NS - 2u);   // later steps whose copies may still be in flight
-        switch (ahead) {
-            case 6: CATCOC_WAIT_VMCNT(6 * STEP_CP); break;
-            case 5: CATCOC_WAIT_VMCNT(5 * STEP_CP); break;
-            case 4: CATCOC_WAIT_VMCNT(4 * STEP_CP); break;
-            case 3: CATCOC_WAIT_VMCNT(3 * STEP_CP); break;
-            case 2: CATCOC_WAIT_VMCNT(2 * STEP_CP); break;
+    // The loop is paced by latencies, not by bandwidth (one wave per SIMD: barrier, LDS round trip and the MFMA
+    // chain of a step add up), so G steps share one barrier and one LDS round trip.  `issued` counts the steps
+    // whose copies have been issued; before a group is read, the copies of later steps may stay in flight.
+    uint32_t issued = umin(nsteps, (uint32_t)(NS - G));
+    for (uint32_t i = 0; i < issued; ++i) issue(i, i);
+    auto wait_steps_in_flight = [&](uint32_t n) {
+        switch (n) {
+            case 0: CATCOC_WAIT_VMCNT(0); break;
             case 1: CATCOC_WAIT_VMCNT(1 * STEP_CP); break;
-            default: CATCOC_WAIT_VMCNT(0); break;
+            case 2: CATCOC_WAIT_VMCNT(2 * STEP_CP); break;
+            case 3: CATCOC_WAIT_VMCNT(3 * STEP_CP); break;
+            case 4: CATCOC_WAIT_VMCNT(4 * STEP_CP); break;
+            case 5: CATCOC_WAIT_VMCNT(5 * STEP_CP); break;
+            case 6: CATCOC_WAIT_VMCNT(6 * STEP_CP); break;
+            case 7: CATCOC_WAIT_VMCNT(7 * STEP_CP); break;
+            default: CATCOC_WAIT_VMCNT(8 * STEP_CP); break;
         }
+    };
+    static_assert(NS - G <= 8 && NS >= 2 * G && NS % G == 0, "ring geometry");
+    auto k_group = [&](uint32_t s, auto count) {   // steps s .. s + GG - 1
+        constexpr int GG = decltype(count)::value;
+        wait_steps_in_flight(issued - (s + GG));
         barrier_keep_vmem();
-        // stage (kt + NS - 1) % NS was read in step kt - 1, which every wave has left
-        if (kt + NS - 1 < nsteps) issue((kt + NS - 1) & (NS - 1), kt + NS - 1);
-        const unsigned char *sa = smem + (kt & (NS - 1)) * STAGE, *sb = sa + A_STAGE;
-        // all fragment reads of the step first, then the MFMAs: one LDS round trip per step instead of one per
-        // 32-row block (left to itself the compiler reuses two fragment registers and serialises them)
-        v4i bf[2], af[2][MBW];
+        // every wave has left the steps before s: their stages take the next copies
+        while (issued < nsteps && issued < s + NS) {
+            issue(issued % NS, issued);
+            ++issued;
+        }
+        // all fragment reads of the group first, then the MFMAs: one LDS round trip per group (left to itself the
+        // compiler reuses two fragment registers and serialises them)
+        v4i bf[GG][2], af[GG][2][MBW];
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-            const unsigned char *p = sb + b_lds + kk * 32 * 128;
-            const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
-            const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 128));
-            bf[kk] = v4i{t0.x, t0.y, t1.x, t1.y};
+        for (int j = 0; j < GG; ++j) {
+            const unsigned char *sa = smem + ((s + j) % NS) * STAGE, *sb = sa + A_STAGE;
 #pragma unroll
-            for (int mb = 0; mb < MBW; ++mb)
-                af[kk][mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
+            for (int kk = 0; kk < 2; ++kk) {
+                const unsigned char *p = sb + b_lds + kk * 32 * 128;
+                const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
+                const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 128));
+                bf[j][kk] = v4i{t0.x, t0.y, t1.x, t1.y};
+#pragma unroll
+                for (int mb = 0; mb < MBW; ++mb)
+                    af[j][kk][mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
+        for (int j = 0; j < GG; ++j)
 #pragma unroll
-            for (int mb = 0; mb < MBW; ++mb) acc[mb] = mfma32<DT_I8>(af[kk][mb], bf[kk], acc[mb]);
+            for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                for (int mb = 0; mb < MBW; ++mb) acc[mb] = mfma32<DT_I8>(af[j][kk][mb], bf[j][kk], acc[mb]);
         __builtin_amdgcn_sched_barrier(0);
-    }
+    };
+    // The groups that still issue copies, then the request for the epilogue's operands (younger than every copy,
+    // so the waits of the remaining groups, which count outstanding operations, stay on the safe side), then the
+    // rest; steps left over by a k slice that is not a multiple of G go one at a time.
+    uint32_t s = 0;
+    for (; issued < nsteps && s + G <= nsteps; s += G) k_group(s, std::integral_constant<int, G>{});
+    request_epilogue_operands();
+    for (; s + G <= nsteps; s += G) k_group(s, std::integral_constant<int, G>{});
+    for (; s < nsteps; ++s) k_group(s, std::integral_constant<int, 1>{});
 
     // ---- k slices meet -------------------------------------------------------------
     if (f > 1) {
