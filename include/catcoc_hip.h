@@ -247,6 +247,10 @@ CATCOC_API void catcoc_splitk_block_coord(uint32_t off, uint32_t dir, uint32_t l
                                           uint32_t kTiles, uint32_t f, uint32_t task, uint32_t *mIdx,
                                           uint32_t *nIdx, uint32_t *kIdx, uint32_t *slice);
 CATCOC_API uint32_t catcoc_splitk_actual_k(uint32_t K, uint32_t k0, uint32_t f, uint32_t slice);
+/* Which task of SplitkGemmIdentityBlockSwizzle workgroup `wg` of a split-K launch runs: a permutation that puts
+ * the row tiles sharing a slice of B on one XCD.  No counterpart in the reference (its cores share one L2). */
+CATCOC_API uint32_t catcoc_splitk_launch_task(uint32_t off, uint32_t dir, uint32_t loopsM, uint32_t loopsN,
+                                              uint32_t f, uint32_t wg);
 /* GemmIdentityBlockSwizzleAllGather::GetBlockCoord (include/catcoc/dgemm/block/block_swizzle_allgather.hpp:88-108). */
 CATCOC_API void catcoc_allgather_block_coord(uint32_t off, uint32_t dir, uint32_t P, uint32_t commInterval,
                                              uint32_t loopsMRank, uint32_t loopsN, uint32_t task, uint32_t *mIdx,

@@ -598,6 +598,11 @@ void catcoc_splitk_block_coord(uint32_t off, uint32_t dir, uint32_t loopsM, uint
 
 uint32_t catcoc_splitk_actual_k(uint32_t K, uint32_t k0, uint32_t f, uint32_t slice) { return splitk_actual_k(K, k0, f, slice); }
 
+uint32_t catcoc_splitk_launch_task(uint32_t off, uint32_t dir, uint32_t loopsM, uint32_t loopsN, uint32_t f, uint32_t wg)
+{
+    return splitk_launch_task(off, dir, loopsM, loopsN, f, wg);
+}
+
 void catcoc_allgather_block_coord(uint32_t off, uint32_t dir, uint32_t P, uint32_t commInterval, uint32_t loopsMRank,
                                   uint32_t loopsN, uint32_t task, uint32_t *mIdx, uint32_t *nIdx)
 {

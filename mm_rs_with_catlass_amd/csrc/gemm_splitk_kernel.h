@@ -51,7 +51,8 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     const uint32_t M = args.M, N = args.N, K = args.K, f = args.splitK;
     const uint32_t loopsM = ceil_div(M, 128u), loopsN = N / 128u, kTiles = ceil_div(K, 256u);
     uint32_t mi, ni, kIdx, slice;
-    splitk_block_coord(args.sched.off, args.sched.dir, loopsM, loopsN, kTiles, f, blockIdx.x, mi, ni, kIdx, slice);
+    const uint32_t task = splitk_launch_task(args.sched.off, args.sched.dir, loopsM, loopsN, f, blockIdx.x);
+    splitk_block_coord(args.sched.off, args.sched.dir, loopsM, loopsN, kTiles, f, task, mi, ni, kIdx, slice);
     const uint32_t kBeg = kIdx * 256u;
     const uint32_t nsteps = splitk_actual_k(K, 256u, f, slice) / 64u;
     const uint32_t row0 = mi * 128u, colT = ni * 128u;

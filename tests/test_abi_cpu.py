@@ -149,6 +149,27 @@ def test_launch_order_is_a_bijection_with_kept_tiles_first_or_last(so):
             assert max(wg for wg in range(n) if kept[wg]) < span
 
 
+def test_splitk_launch_order_is_a_permutation_that_groups_b_readers(so):
+    import ctypes as C
+    for loopsM, loopsN, f in [(1, 64, 4), (4, 64, 1), (2, 16, 3), (1, 8, 1), (3, 24, 2), (1, 3, 4), (2, 5, 1)]:
+        total = loopsM * loopsN * f
+        tasks = [so.catcoc_splitk_launch_task(7, 1, loopsM, loopsN, f, wg) for wg in range(total)]
+        assert sorted(tasks) == list(range(total))
+        assert so.catcoc_splitk_launch_task(7, 1, loopsM, loopsN, f, total + 5) == total + 5
+        if (loopsN * f) % 8 or loopsM < 2:
+            assert tasks == list(range(total))      # the order does not apply: identity
+            continue
+        m, n, k, sl = (C.c_uint32() for _ in range(4))
+        where = {}
+        for wg, task in enumerate(tasks):
+            so.catcoc_splitk_block_coord(7, 1, loopsM, loopsN, 32, f, task, C.byref(m), C.byref(n), C.byref(k), C.byref(sl))
+            where.setdefault((n.value, sl.value), []).append(wg)
+        for wgs in where.values():
+            # the loopsM row tiles that stream one (column tile, k slice) of B sit on one XCD, dispatched back to back
+            assert len(wgs) == loopsM and len({w % 8 for w in wgs}) == 1
+            assert max(wgs) - min(wgs) == 8 * (loopsM - 1)
+
+
 def test_workspace_size_queries(so):
     from mm_rs_with_catlass_amd import ops
     need, f, tiles = ops.splitk_plan(16, 8192, 8192, 8, 0, 2)
