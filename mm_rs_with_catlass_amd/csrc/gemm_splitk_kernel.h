@@ -315,9 +315,10 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         const uint32_t vrel = mb * 32 + 4u * h;   // slot r is a row of A when slot_row(r) + vrel < rowsValid
         int iv[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            iv[r] = acc[mb][r] + bv;
-            csum += (slot_row(r) + vrel < rowsValid && !lane_kept(k, r)) ? iv[r] : 0;
+        for (int r = 0; r < 16; ++r) iv[r] = acc[mb][r] + bv;
+        if (args.checksum != nullptr) {   // rows that are not kept are only summed, and only on request
+#pragma unroll
+            for (int r = 0; r < 16; ++r) csum += (slot_row(r) + vrel < rowsValid && !lane_kept(k, r)) ? iv[r] : 0;
         }
         if (args.accDump) {
 #pragma unroll
