@@ -458,6 +458,50 @@ def test_quant_config4_full_size_properties():
 
 
 # ------------------------------------------------------- C ABI from a plain C++ host
+def test_launches_replay_from_a_hip_graph():
+    # serving loops capture their launches: the library allocates nothing and never synchronises, the split-K path
+    # re-arms its counters inside the kernel, so a captured launch replays; every replay must equal the eager result
+    _need_gpu()
+    g = torch.Generator(device=DEV).manual_seed(5)
+    M, K, N, P = 1024, 512, 512, 4
+    x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
+    x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=DEV, generator=g)
+    s1 = torch.empty(M, device=DEV).uniform_(0.005, 0.02, generator=g)
+    s2 = torch.empty(N, device=DEV).uniform_(0.001, 0.01, generator=g)
+    peers = [torch.randn((M // P, N), device=DEV, generator=g) for _ in range(P - 1)]
+    big, out_big = ops.prepare_quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, 1, P)
+    xs = torch.randint(-127, 128, (16, 2048), dtype=torch.int8, device=DEV, generator=g)
+    w = torch.randint(-127, 128, (2048, 512), dtype=torch.int8, device=DEV, generator=g)
+    ss = torch.empty(16, device=DEV).uniform_(0.005, 0.02, generator=g)
+    pk = [torch.randn((2, N), device=DEV, generator=g) for _ in range(P - 1)]
+    need, fac, tiles = ops.splitk_plan(16, 2048, 512, P, 4, 2, split_k=4)
+    assert fac == 4
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    small, out_small = ops.prepare_quant_matmul_splitk(xs, w, ss, s2, None, pk, P, 4, 2, split_k=4, workspace=ws)
+    big(); small(); L.check()
+    torch.cuda.synchronize()
+    want_big, want_small = out_big.clone(), out_small.clone()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        big(); small()                       # warm the side stream before capture
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            out_big.zero_()
+            out_small.zero_()
+            big()
+            small()
+    L.check()
+    for _ in range(3):
+        out_big.fill_(1.0)                   # eager work between the replays
+        out_small.fill_(1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_big, want_big) and torch.equal(out_small, want_small)
+        assert not ws[tiles * fac * 128 * 128 * 4:].any(), "tile counters were not re-armed"
+
+
 def test_cpp_host_drives_the_library_through_the_c_abi(tmp_path):
     # the stand-alone host (no Python, no torch in the process) reads the reference's raw .bin files, launches
     # catcoc_quant_matmul_reduce_scatter and writes this rank's block of output.bin at its offset
