@@ -131,6 +131,11 @@ def float_configs(args, torch, L, ops, dev):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / args.steps, e0.elapsed_time(e1) / args.steps / 1e3
 
+    def slices(comm, dt, m, k, n, rank, p):
+        """Workspace for a launch of few tiles (the library cuts their k range into slices that meet through it)."""
+        need, f = ops.kslice_plan(comm, dt, m, k, n, rank, p)
+        return (torch.zeros(need, dtype=torch.uint8, device=dev) if f > 1 else None), f
+
     res = []
     # config 3: fp16 matmul-reduce-scatter, A[4096,1792] N(0,1), B[1792,4096] N(0,0.02), 7 fp32 peers, keep [512,4096]
     M, K, N, P, rank = 4096, 1792, 4096, 8, 0
@@ -153,18 +158,20 @@ def float_configs(args, torch, L, ops, dev):
     shards = [torch.randn((m, K), device=dev, generator=g).bfloat16() for _ in range(P)]
     B2 = (torch.randn((K, N), device=dev, generator=g) * 0.02).bfloat16()
     out2 = torch.empty((m * P, N), dtype=torch.bfloat16, device=dev)
-    wall, kern = timed(lambda: ops.allgather_matmul(shards[0], shards[1:], B2, 0, P, out=out2))
+    ws2, f2 = slices(L.ALLGATHER_MATMUL, torch.bfloat16, m, K, N, 0, P)
+    wall, kern = timed(lambda: ops.allgather_matmul(shards[0], shards[1:], B2, 0, P, out=out2, workspace=ws2))
     res.append({"config": 2, "op": "allgather_matmul bf16 8 x [512,4096] x [4096,1024]", "kernel_us": round(kern * 1e6, 2),
-                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * m * P * N * K / kern / 1e12, 1)})
+                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * m * P * N * K / kern / 1e12, 1), "k_slices": f2})
     # config 1: fp16 all-reduce share, A[512,1024] (this rank's k half), B[1024,1024], one fp32 peer
     M, K, N, P = 512, 1024, 1024, 2
     A1 = (torch.rand((M, K), device=dev, generator=g) * 2 - 1).half()
     B1 = (torch.rand((K, N), device=dev, generator=g) * 2 - 1).half()
     peer = [torch.randn((M, N), device=dev, generator=g)]
     out1 = torch.empty((M, N), dtype=torch.float16, device=dev)
-    wall, kern = timed(lambda: ops.matmul_allreduce(A1, B1, peer, 0, P, out=out1))
+    ws1, f1 = slices(L.MATMUL_ALLREDUCE, torch.float16, M, K, N, 0, P)
+    wall, kern = timed(lambda: ops.matmul_allreduce(A1, B1, peer, 0, P, out=out1, workspace=ws1))
     res.append({"config": 1, "op": "matmul_allreduce fp16 M=512 K=1024(local) N=1024 P=2", "kernel_us": round(kern * 1e6, 2),
-                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * M * N * K / kern / 1e12, 1)})
+                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * M * N * K / kern / 1e12, 1), "k_slices": f1})
     c3 = res[0]
     print(json.dumps({
         "metric": "fp16 matmul-reduce-scatter shard (BASELINE config 3) TFLOPS, 1 MI355X", "value": c3["TFLOPS"], "unit": "TFLOPS",

@@ -113,7 +113,8 @@ typedef struct CatcocSymmetricDesc {
     uint32_t keptRowBegin;    /* keptRows == 0: the rank keeps rows [rankIdx*m/rankSize, +m/rankSize) as in the reference. */
     uint32_t keptRows;        /* keptRows != 0 (W8A8 only): the rank keeps rows [keptRowBegin, +keptRows) of an m that need not
                                  divide by rankSize, and the launch takes the skinny-M split-K path (decode shapes) */
-    uint32_t splitK;          /* split-K path: k slices per tile; 0 = GetSplitkFactor with blockNum cores and 128x128x256 tiles */
+    uint32_t splitK;          /* k slices per tile; 0 = the library's choice (split-K path: GetSplitkFactor with blockNum cores
+                                 and 128x128x256 tiles; large-tile kernel: see catcoc_get_kslice_workspace_size) */
     /* Reduce paths: peers[s], s = 0..rankSize-2, are the other ranks' partial
      * results for this rank's kept rows (fp32, or int32 with REDUCE_INT32), added
      * in slot order after the local partial.  Row `peerRowOffset + i` of a peer
@@ -127,9 +128,11 @@ typedef struct CatcocSymmetricDesc {
     uint64_t outboundBytes;   /* capacity of `outbound` */
     int64_t *checksum;        /* OUTBOUND_CHECKSUM target: one int64 per task (W8A8) / one double per task (float) */
     void *accDump;            /* optional full [m,n] int32 (W8A8) or fp32 (float) local partial, for bit-exact checks */
-    /* Split-K path only: int32 partial tiles and tile counters, catcoc_get_splitk_workspace_size() bytes,
-     * 256-byte aligned, ZEROED by the caller once before its first use (the library leaves it re-armed after
-     * every launch).  Launches that share a workspace must not overlap (same stream, or ordered by events). */
+    /* Scratch in HBM for launches whose k range is cut into slices: the skinny-M split-K path
+     * (catcoc_get_splitk_workspace_size() bytes) and few-tile launches of the large-tile kernel
+     * (catcoc_get_kslice_workspace_size() bytes, optional there).  256-byte aligned, ZEROED by the caller once
+     * before its first use (the library leaves it re-armed after every launch).  Launches that share a workspace
+     * must not overlap (same stream, or ordered by events). */
     void *workspace;
     uint64_t workspaceBytes;
 } CatcocSymmetricDesc;
@@ -201,6 +204,18 @@ CATCOC_API int catcoc_can_implement(int commType, int dataType, const CocTilingP
  * sizes layoutSymmetric = m0*commInterval*BLOCK_NUM*WORKSPACE_STAGES x n0, matmul_reduce_scatter.h:161). */
 CATCOC_API uint64_t catcoc_get_workspace_size(int commType, int dataType, const CocTilingParams *tiling,
                                               const CatcocSymmetricDesc *desc);
+
+/* Launches with few 128x256 tiles (fewer than half the CUs' worth) can cut every tile's k range into k slices, one
+ * workgroup each, that meet through `workspace` (partial tiles in 32-bit words + one counter per tile, zeroed once
+ * by the caller, re-armed by every launch): returns the bytes needed and the slice count (1 and 0 bytes when the
+ * launch would not be sliced: other tile shapes, transposed or ragged operands, enough tiles already).  The count
+ * is 2, 4 or 8 for W8A8 (integer partials add exactly) and at most 2 for fp16/bf16 (a two-term fp32 sum does not
+ * depend on which slice arrives last); desc->splitK, when non-zero, is taken as the caller's own count.  A launch
+ * slices only when `workspace` is given.  Counterpart in the reference: SplitkMatmul's k split
+ * (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:68-148), which its communication kernels do not
+ * use. */
+CATCOC_API uint64_t catcoc_get_kslice_workspace_size(int commType, int dataType, const CocTilingParams *tiling,
+                                                     const CatcocSymmetricDesc *desc, uint32_t *kSlices);
 
 /* Split-K path (descriptor with keptRows != 0): bytes of `workspace` the launch needs (0 when the split factor
  * is 1), the split factor it will use and its number of 128x128 tiles (`checksum`, if given, needs one int64 per

@@ -65,6 +65,8 @@ struct Plan {
     uint32_t dtype;
     uint32_t blockNum;
     bool dma;     // full tiles, row-major operands: the direct-to-LDS kernel applies
+    uint32_t kSlices;        // k slices per tile this launch would run with a workspace (1 = none)
+    uint64_t kSliceBytes;    // workspace for that: partial tiles + counters
 };
 
 uint32_t elem_size(uint32_t dt) { return dt == DT_I8 ? 1u : 2u; }
@@ -189,6 +191,40 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
         a.checksum = d->checksum;
     }
     a.accDump = d->accDump;
+
+    // Few tiles: the 128-row direct-to-LDS kernel can cut every tile's k range into slices, one workgroup each, that
+    // meet through a workspace (partial tiles [tiles][slices][128*256] as 32-bit words, then one counter per tile).
+    // Chosen so that the slices fill the 256 CUs once, each with at least eight k steps; float partials are limited to
+    // two slices (their sum does not depend on which arrives last).  desc.splitK overrides the choice.
+    plan.kSlices = 1;
+    plan.kSliceBytes = 0;
+    if (plan.dma && m0 == 128 && d->keptRows == 0) {
+        const uint32_t T = a.sched.coreLoops, nkAll = (uint32_t)((uint64_t)t->k * es / 64u);
+        const uint32_t fmax = dt == DT_I8 ? 8u : 2u;
+        uint32_t f = 1;
+        if (d->splitK != 0) {
+            if (d->splitK > fmax || d->splitK > nkAll)
+                return fail(E_TILING, "splitK %u: at most %u k slices for this element type and k", d->splitK, umin(fmax, nkAll));
+            f = d->splitK;
+        } else {
+            while (f * 2u <= fmax && T * f * 2u <= 256u && nkAll / (f * 2u) >= 8u) f *= 2u;
+        }
+        if (f > 1) {
+            plan.kSlices = f;
+            plan.kSliceBytes = (uint64_t)T * f * (128u * 256u * 4u) + (((uint64_t)T * 4u + 255u) & ~255ull);
+            if (d->workspace != nullptr) {
+                if ((uintptr_t)d->workspace % 256 != 0) return fail(E_WORKSPACE, "workspace must be 256-byte aligned");
+                if (d->workspaceBytes < plan.kSliceBytes)
+                    return fail(E_WORKSPACE, "workspace too small for %u k slices: %llu < %llu bytes", f,
+                                (unsigned long long)d->workspaceBytes, (unsigned long long)plan.kSliceBytes);
+                a.splitK = f;
+                a.skPart = (int32_t *)d->workspace;
+                a.skCount = (uint32_t *)((unsigned char *)d->workspace + (uint64_t)T * f * (128u * 256u * 4u));
+            } else if (d->splitK != 0) {
+                return fail(E_WORKSPACE, "splitK %u needs a workspace of %llu bytes", f, (unsigned long long)plan.kSliceBytes);
+            }
+        }
+    }
     return 0;
 }
 
@@ -217,6 +253,7 @@ void launch_float(int commType, int dataType, void *stream, uint8_t *a, uint8_t 
     p.args.d = c;
     if (!check_ptr_align(p, a, b)) p.variant = 0;
     const bool dma = p.dma && p.variant != 0 && (uintptr_t)b % 16 == 0 && (p.args.ldb * 2) % 16 == 0 && (uintptr_t)c % 16 == 0;
+    if (!dma) p.args.splitK = 0;   // the other kernels run every tile whole
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles and 16-byte aligned row-major operands"); return; }
     const int e = dma ? (p.dtype == DT_F16 ? launch_gemm_dma_f16(p.args, stream) : launch_gemm_dma_bf16(p.args, stream))
                       : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
@@ -350,6 +387,7 @@ void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uin
     bool dma = p.dma && p.variant != 0 && (uintptr_t)x2 % 16 == 0 && p.args.ldb % 16 == 0 && (uintptr_t)d_out % 16 == 0;
     for (uint32_t s = 0; s < p.args.nPeers && dma; ++s) dma = (uintptr_t)p.args.peers[s] % 16 == 0;
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles, 16-byte aligned row-major operands and fp32 peers"); return; }
+    if (!dma) p.args.splitK = 0;   // the other kernels run every tile whole
     const int e = dma ? launch_gemm_dma_i8(p.args, stream) : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
     ok();
@@ -436,6 +474,29 @@ uint64_t catcoc_get_workspace_size(int commType, int dataType, const CocTilingPa
     if (make_plan(commType, dataType, tiling, &d, 0, 0, p)) return 0;
     ok();
     return (uint64_t)p.args.sched.stages * p.args.sched.blockPerComm * p.args.sched.m0 * p.args.sched.n0 * 4u;
+}
+
+uint64_t catcoc_get_kslice_workspace_size(int commType, int dataType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
+                                          uint32_t *kSlices)
+{
+    Plan p;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
+    d = *desc;
+    d.flags &= ~CATCOC_OUTBOUND_MASK;
+    d.workspace = nullptr;
+    const uint32_t forced = d.splitK;
+    d.splitK = 0;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    if (forced != 0) {   // size for the caller's own slice count: plan it with a workspace that is large enough
+        d.splitK = forced;
+        d.workspace = (void *)256;
+        d.workspaceBytes = ~0ull;
+    }
+    if (make_plan(commType, dataType, tiling, &d, 0, 0, p)) return 0;
+    ok();
+    if (kSlices) *kSlices = p.kSlices;
+    return p.kSliceBytes;
 }
 
 uint64_t catcoc_get_splitk_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t *splitK,

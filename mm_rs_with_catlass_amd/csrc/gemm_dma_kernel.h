@@ -103,7 +103,21 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 
     const SchedParams &sp = args.sched;
     const bool linear = (args.flags & GF_LINEAR_ORDER) != 0;
-    const uint32_t task = launch_task(sp, blockIdx.x, linear, args.keptRank);
+    // A launch with few tiles can cut every tile's k range into kSlices pieces, one workgroup each (128-row tiles
+    // only): position `pos` of the launch order runs as kSlices workgroups that stay in the position's XCD column.
+    uint32_t pos = blockIdx.x, slice = 0;
+    const uint32_t kSlices = (WM == 2 && args.splitK > 1) ? args.splitK : 1u;
+    if (kSlices > 1) {
+        if ((sp.coreLoops & 7u) == 0) {
+            const uint32_t q = blockIdx.x >> 3;
+            slice = q % kSlices;
+            pos = (q / kSlices) * 8u + (blockIdx.x & 7u);
+        } else {
+            slice = blockIdx.x % kSlices;
+            pos = blockIdx.x / kSlices;
+        }
+    }
+    const uint32_t task = launch_task(sp, pos, linear, args.keptRank);
     TileInfo ti;
     if (!task_tile(sp, task, ti)) return;
     // The kept tiles are the longest chain of a reduce-scatter launch (main loop, then the peers' partials):
@@ -116,6 +130,12 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const unsigned char *Ag = (const unsigned char *)args.a[gather ? ti.targetRank : 0] +
                               (int64_t)(gather ? ti.rowInRank : ti.row) * ldaB;
     const unsigned char *Bg = (const unsigned char *)args.b + (size_t)ti.col * ES;
+    // k steps (64 bytes of K each) of this workgroup: all of them, or its slice
+    const uint32_t nkAll = args.K * ES / 64;
+    const uint32_t kFirst = (uint32_t)(((uint64_t)nkAll * slice) / kSlices);
+    const uint32_t nk = (uint32_t)(((uint64_t)nkAll * (slice + 1u)) / kSlices) - kFirst;
+    Ag += (size_t)kFirst * 64;
+    Bg += (size_t)kFirst * (64 / ES) * ldbB;
 
     // ---- copy descriptors ---------------------------------------------------
     // Every copy a wave issues has its own global pointer, advanced after each issue, and a scalar LDS address:
@@ -272,7 +292,6 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 #undef CATCOC_MMA
     auto nothing = [] {};
 
-    const uint32_t nk = args.K * ES / 64;
     if constexpr (BM == 128) {
         // ---- 3 stages, copies run two k steps ahead (72 KiB LDS, two workgroups per CU) ----
         auto stA = [&](uint32_t s3) { return smem + s3 * A_STAGE; };
@@ -425,6 +444,69 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     }
 
 #undef CATCOC_FENCE
+
+    // ---- k slices meet --------------------------------------------------------------
+    // Every slice writes its partial tile through to memory (device-scope stores, 16 bytes per lane, the tile in
+    // register order: index (((mb*4 + nb)*4 + g)*256 + thread)*4 + j holds register r = 4g + j), a per-tile counter
+    // elects the last slice to arrive, and that workgroup adds the others' partials and goes on to the epilogue.
+    // Integer partials add exactly in any order; float partials are limited to two slices by the host, whose sum
+    // does not depend on which of them arrives last.
+    if constexpr (WM == 2) {
+        if (kSlices > 1) {
+            constexpr int DEVICE_SCOPE = 16;   // sc1
+            constexpr uint32_t TILE_WORDS = 128 * 256;
+            const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(args.skPart + ((size_t)task * kSlices + slice) * TILE_WORDS), 0, (int)(TILE_WORDS * 4), 0x00020000);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const auto e0 = acc[mb][nb][4 * g], e1 = acc[mb][nb][4 * g + 1], e2 = acc[mb][nb][4 * g + 2], e3 = acc[mb][nb][4 * g + 3];
+                        const v4i iv = {__builtin_bit_cast(int, e0), __builtin_bit_cast(int, e1), __builtin_bit_cast(int, e2), __builtin_bit_cast(int, e3)};
+                        __builtin_amdgcn_raw_buffer_store_b128(iv, mine, (((mb * 4 + nb) * 4 + g) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+                    }
+            CATCOC_WAIT_VMCNT(0);   // once the stores are acknowledged the slice may be counted
+            __syncthreads();
+            volatile uint32_t *flag = (volatile uint32_t *)smem;
+            if (tid == 0) *flag = __hip_atomic_fetch_add(args.skCount + task, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            if (*flag != kSlices - 1u) return;
+            if (tid == 0) __hip_atomic_store(args.skCount + task, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (uint32_t o = 0; o + 1 < kSlices; ++o) {
+                const uint32_t sl = o < slice ? o : o + 1;
+                const __amdgpu_buffer_rsrc_t other = __builtin_amdgcn_make_buffer_rsrc(
+                    (void *)(args.skPart + ((size_t)task * kSlices + sl) * TILE_WORDS), 0, (int)(TILE_WORDS * 4), 0x00020000);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {   // one 32-row block (64 registers) per round trip
+                    v4i pv[4][4];
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g)
+                            pv[nb][g] = __builtin_amdgcn_raw_buffer_load_b128(other, (((mb * 4 + nb) * 4 + g) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const int p0 = pv[nb][g].x, p1 = pv[nb][g].y, p2 = pv[nb][g].z, p3 = pv[nb][g].w;
+                            if constexpr (DT == DT_I8) {
+                                acc[mb][nb][4 * g] += p0;
+                                acc[mb][nb][4 * g + 1] += p1;
+                                acc[mb][nb][4 * g + 2] += p2;
+                                acc[mb][nb][4 * g + 3] += p3;
+                            } else {
+                                acc[mb][nb][4 * g] += __builtin_bit_cast(float, p0);
+                                acc[mb][nb][4 * g + 1] += __builtin_bit_cast(float, p1);
+                                acc[mb][nb][4 * g + 2] += __builtin_bit_cast(float, p2);
+                                acc[mb][nb][4 * g + 3] += __builtin_bit_cast(float, p3);
+                            }
+                        }
+                }
+            }
+        }
+    }
 
     // ---- epilogue -----------------------------------------------------------------
     // acc[mb][nb][r] is element (row, col) of the tile with

@@ -12,11 +12,11 @@ int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream)
 // m0 = 128 (4 waves, two workgroups per CU) or m0 = 256 (8 waves).
 int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
 {
-    const dim3 grid(args.sched.coreLoops);
     if (args.sched.m0 == 256)
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), grid, dim3(512), 0, (hipStream_t)stream, args);
-    else
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2>), grid, dim3(256), 0, (hipStream_t)stream, args);
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), dim3(args.sched.coreLoops), dim3(512), 0, (hipStream_t)stream, args);
+    else   // one workgroup per tile, or per k slice of a tile
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2>), dim3(args.sched.coreLoops * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
+                           (hipStream_t)stream, args);
     return (int)hipGetLastError();
 }
 }  // namespace catcoc

@@ -60,7 +60,7 @@ EXPORTS = [
     "catcoc_launch_matmul_reduce_scatter_fp16", "catcoc_launch_matmul_reduce_scatter_bf16",
     "catcoc_quant_matmul_reduce_scatter", "catcoc_launch_quant_matmul_reduce_scatter",
     "catcoc_last_error", "catcoc_last_status", "catcoc_can_implement", "catcoc_get_workspace_size",
-    "catcoc_get_splitk_workspace_size",
+    "catcoc_get_splitk_workspace_size", "catcoc_get_kslice_workspace_size",
     "catcoc_get_task_count", "catcoc_get_tilings", "catcoc_check_comm_interval_reduce_scatter",
     "catcoc_check_comm_interval_allreduce", "catcoc_check_comm_interval_allgather", "catcoc_get_splitk_factor",
     "catcoc_default_tiling", "catcoc_swizzle_block_coord", "catcoc_splitk_block_coord", "catcoc_splitk_actual_k", "catcoc_splitk_launch_task",
@@ -123,6 +123,8 @@ def load():
     L.catcoc_can_implement.restype = C.c_int
     L.catcoc_get_workspace_size.argtypes = [C.c_int, C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc)]
     L.catcoc_get_workspace_size.restype = C.c_uint64
+    L.catcoc_get_kslice_workspace_size.argtypes = [C.c_int, C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), pu]
+    L.catcoc_get_kslice_workspace_size.restype = C.c_uint64
     L.catcoc_get_splitk_workspace_size.argtypes = [C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), pu, pu]
     L.catcoc_get_splitk_workspace_size.restype = C.c_uint64
     L.catcoc_launch_task.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32]

@@ -47,6 +47,15 @@ def _check_dev(*ts):
             raise _l.CatcocError("operands must be contiguous")
 
 
+def _attach_workspace(d, workspace, split_k):
+    """Optional scratch for k-sliced launches (kslice_plan() says how large) and the caller's own slice count."""
+    d.splitK = split_k
+    if workspace is not None:
+        _check_dev(workspace)
+        d.workspace = workspace.data_ptr()
+        d.workspaceBytes = workspace.numel() * workspace.element_size()
+
+
 def _desc(rank, rank_size, peers, peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump):
     peer_ld = peers[0].shape[1] if peers else 0
     return _l.make_desc(
@@ -59,7 +68,7 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
                                         out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
                                         reduce_int32=False, outbound=None, checksum=None, acc_dump=None,
                                         c_accum=None, block_num=0, stages=0, swizzle=None, linear_order=False,
-                                        out=None):
+                                        out=None, workspace=None, split_k=0):
     """Validate and bind the arguments once; returns (launch, out) where launch() enqueues one call of
     catcoc_launch_quant_matmul_reduce_scatter on torch's current stream (for launch-rate-sensitive loops)."""
     _check_dev(x1, x2, scale_x1, scale_x2, bias, outbound, checksum, acc_dump, c_accum, *peers)
@@ -69,10 +78,11 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
     flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_REDUCE_INT32 if reduce_int32 else 0) | \
         (_l.FLAG_LINEAR_ORDER if linear_order else 0)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
+    _attach_workspace(d, workspace, split_k)
     if out is None:
         out = torch.empty((m // max(rank_size, 1), n), dtype=out_dtype, device=x1.device)
     L = _l.load()
-    keep = (x1, x2, scale_x1, scale_x2, bias, tuple(peers), outbound, checksum, acc_dump, c_accum, out, d, t)
+    keep = (x1, x2, scale_x1, scale_x2, bias, tuple(peers), outbound, checksum, acc_dump, c_accum, out, d, t, workspace)
     fn = L.catcoc_launch_quant_matmul_reduce_scatter
     argv = (0, x1.data_ptr(), x2.data_ptr(), scale_x1.data_ptr(), scale_x2.data_ptr(), _ptr(bias), _ptr(c_accum),
             out.data_ptr(), C.addressof(d), C.byref(t), 0, int(trans_b), _TORCH_TO_DT[out.dtype])
@@ -86,17 +96,19 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
 def quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(), rank=0, rank_size=1,
                                 out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
                                 reduce_int32=False, outbound=None, checksum=None, acc_dump=None, c_accum=None,
-                                block_num=0, stages=0, swizzle=None, linear_order=False, out=None):
+                                block_num=0, stages=0, swizzle=None, linear_order=False, out=None, workspace=None,
+                                split_k=0):
     """W8A8 matmul -> reduce-scatter share of one rank.
 
     x1 [m,k] int8, x2 [k,n] int8 ([n,k] with trans_b), scale_x1 [m] fp32 per token, scale_x2 [n] fp32 per
     channel, bias [n] int32 or None.  peers: rank_size-1 staged partials for the kept rows (fp32, or int32
-    with reduce_int32), added in list order after the local partial.
+    with reduce_int32), added in list order after the local partial.  workspace: optional zero-initialised uint8
+    tensor of kslice_plan() bytes with which a launch of few tiles cuts its k range into slices.
     Returns d_out [m/rank_size, n].
     """
     launch, out = prepare_quant_matmul_reduce_scatter(
         x1, x2, scale_x1, scale_x2, bias, peers, rank, rank_size, out_dtype, tiling, trans_b, peer_row_offset,
-        reduce_int32, outbound, checksum, acc_dump, c_accum, block_num, stages, swizzle, linear_order, out)
+        reduce_int32, outbound, checksum, acc_dump, c_accum, block_num, stages, swizzle, linear_order, out, workspace, split_k)
     launch()
     _l.check()
     return out
@@ -151,7 +163,7 @@ def quant_matmul_splitk(*args, **kw):
 
 
 def _float_op(comm_type, a, b, c_shape, peers, rank, rank_size, tiling, trans_a, trans_b, peer_row_offset, outbound,
-              checksum, acc_dump, block_num, stages, swizzle, linear_order, out, m_for_tiling):
+              checksum, acc_dump, block_num, stages, swizzle, linear_order, out, m_for_tiling, workspace=None, split_k=0):
     _check_dev(a, b, outbound, checksum, acc_dump, *peers)
     if a.dtype not in _TORCH_TO_DT or b.dtype != a.dtype:
         raise _l.CatcocError("a and b must both be float16 or both bfloat16")
@@ -160,6 +172,7 @@ def _float_op(comm_type, a, b, c_shape, peers, rank, rank_size, tiling, trans_a,
     t = tiling if tiling is not None else default_tiling(m_for_tiling, k, n, rank_size, m0=0, n0=0, k0=0)
     flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_LINEAR_ORDER if linear_order else 0)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
+    _attach_workspace(d, workspace, split_k)
     if out is None:
         out = torch.empty(c_shape(n), dtype=a.dtype, device=a.device)
     L = _l.load()
@@ -174,30 +187,43 @@ def _float_op(comm_type, a, b, c_shape, peers, rank, rank_size, tiling, trans_a,
 
 def matmul_reduce_scatter(a, b, peers=(), rank=0, rank_size=1, tiling=None, trans_a=False, trans_b=False,
                           peer_row_offset=0, outbound=None, checksum=None, acc_dump=None, block_num=0, stages=0,
-                          swizzle=None, linear_order=False, out=None):
+                          swizzle=None, linear_order=False, out=None, workspace=None, split_k=0):
     """fp16/bf16 matmul -> reduce-scatter share: a [m,k], b [k,n], peers fp32; returns [m/rank_size, n]."""
     m = a.shape[1] if trans_a else a.shape[0]
     return _float_op(_l.MATMUL_REDUCE_SCATTER, a, b, lambda n: (m // max(rank_size, 1), n), peers, rank, rank_size,
                      tiling, trans_a, trans_b, peer_row_offset, outbound, checksum, acc_dump, block_num, stages,
-                     swizzle, linear_order, out, m)
+                     swizzle, linear_order, out, m, workspace, split_k)
 
 
 def matmul_allreduce(a, b, peers=(), rank=0, rank_size=1, tiling=None, trans_a=False, trans_b=False,
                      peer_row_offset=0, acc_dump=None, block_num=0, stages=0, swizzle=None, linear_order=False,
-                     out=None):
+                     out=None, workspace=None, split_k=0):
     """fp16/bf16 matmul -> all-reduce share: every row is kept; peers are full [m,n] fp32 partials."""
     m = a.shape[1] if trans_a else a.shape[0]
     return _float_op(_l.MATMUL_ALLREDUCE, a, b, lambda n: (m, n), peers, rank, rank_size, tiling, trans_a, trans_b,
-                     peer_row_offset, None, None, acc_dump, block_num, stages, swizzle, linear_order, out, m)
+                     peer_row_offset, None, None, acc_dump, block_num, stages, swizzle, linear_order, out, m, workspace, split_k)
 
 
 def allgather_matmul(a_local, peer_shards, b, rank=0, rank_size=1, tiling=None, trans_b=False, acc_dump=None,
-                     block_num=0, stages=0, swizzle=None, linear_order=False, out=None):
+                     block_num=0, stages=0, swizzle=None, linear_order=False, out=None, workspace=None, split_k=0):
     """all-gather -> matmul: a_local [m,k] is this rank's shard, peer_shards the other ranks' shards in
     ascending rank order (separate buffers, read in place); returns [m*rank_size, n]."""
     m = a_local.shape[0]
     return _float_op(_l.ALLGATHER_MATMUL, a_local, b, lambda n: (m * rank_size, n), peer_shards, rank, rank_size,
-                     tiling, False, trans_b, 0, None, None, acc_dump, block_num, stages, swizzle, linear_order, out, m)
+                     tiling, False, trans_b, 0, None, None, acc_dump, block_num, stages, swizzle, linear_order, out, m,
+                     workspace, split_k)
+
+
+def kslice_plan(comm_type, dtype, m, k, n, rank=0, rank_size=1, tiling=None, split_k=0):
+    """(workspace bytes, k slices) with which a launch of this shape would cut its tiles' k range; (0, 1) = it would not.
+    m is the first dimension the operator's tiling takes (all-gather: one shard's rows)."""
+    t = tiling if tiling is not None else default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
+    d = _l.make_desc(rank, rank_size)
+    d.splitK = split_k
+    f = C.c_uint32(1)
+    need = int(_l.load().catcoc_get_kslice_workspace_size(comm_type, _TORCH_TO_DT.get(dtype, _l.INT8), C.byref(t), C.byref(d), C.byref(f)))
+    _l.check()
+    return need, f.value
 
 
 def device_info():

@@ -47,7 +47,7 @@ TORCH_DT = {oracle.FP16: torch.float16, oracle.BF16: torch.bfloat16}
 
 def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, trans_b=False, reduce_int32=False,
                full_peers=False, tiling=None, outbound=False, block_num=0, stages=0, swizzle=None, linear=False,
-               launches=1):
+               launches=1, kslices=None):
     _need_gpu()
     x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
     x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
@@ -81,6 +81,15 @@ def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, tran
     checksum = torch.zeros(ntasks, dtype=torch.int64, device=DEV)
     if not outbound:
         kw["checksum"] = checksum
+    ws = None
+    if kslices is not None:      # (forced count or 0 = the library's choice, count expected)
+        need, f = ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, M, K, N, rank, P, tiling=tiling, split_k=kslices[0])
+        assert f == kslices[1]
+        assert need == (ntasks * f * 128 * 256 * 4 + -(-ntasks * 4 // 256) * 256 if f > 1 else 0)
+        if f > 1:
+            ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+            kw["workspace"] = ws
+        kw["split_k"] = kslices[0]
     for it in range(launches):
         out = ops.quant_matmul_reduce_scatter(
             dev(x1), x2d, dev(s1), dev(s2), dev(b) if bias else None, dpeers, rank, P, out_dtype=TORCH_DT[out_dtype],
@@ -89,6 +98,8 @@ def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, tran
         torch.cuda.synchronize()
         if it + 1 < launches:
             out.zero_()
+    if ws is not None:
+        assert not ws[ntasks * kslices[1] * 128 * 256 * 4:].any(), "tile counters were not re-armed"
     acc_got = acc_dump.cpu().numpy()
     assert np.array_equal(acc_got, acc_want), "int32 accumulators differ from the oracle"
     kept = acc_want[rank * rows:(rank + 1) * rows]
@@ -161,6 +172,38 @@ def test_quant_rs_many_tiles_two_launches(case):
     # must rewrite the zeroed output
     M, N, K, P, rank = case
     quant_case(np.random.default_rng(40 + rank), M, N, K, P, rank, bias=True, launches=2)
+
+
+@pytest.mark.parametrize("case", [(1024, 1024, 4096, 4, 1, (0, 8)), (1024, 1024, 2048, 4, 3, (0, 4)), (2048, 512, 1792, 8, 7, (0, 2)),
+                                  (1024, 512, 1024, 2, 0, (3, 3)), (2048, 1024, 576, 8, 3, (0, 1)), (1024, 768, 64, 4, 2, (1, 1))])
+def test_quant_rs_few_tiles_k_sliced(case):
+    # fewer tiles than CUs: with a workspace every tile's k range is cut into slices that meet through memory;
+    # int32 partials add exactly, so everything stays bit-exact, and the second launch finds the counters re-armed
+    M, N, K, P, rank, ks = case
+    r = quant_case(np.random.default_rng(70 + rank), M, N, K, P, rank, bias=True, launches=2, kslices=ks)
+    cs = r["checksum"].cpu().numpy()
+    rows = M // P
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    import ctypes as C
+    tr, row, col = C.c_uint32(), C.c_uint32(), C.c_uint32()
+    for task in range(r["ntasks"]):
+        L.load().catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row), C.byref(col), None)
+        if tr.value != rank:
+            blk = r["acc"][row.value:row.value + 128, col.value:col.value + 256].astype(np.int64)
+            assert cs[task] == blk.sum(), task
+
+
+def test_k_slice_rejections():
+    _need_gpu()
+    a = torch.zeros((512, 1024), dtype=torch.float16, device=DEV)
+    b = torch.zeros((1024, 1024), dtype=torch.float16, device=DEV)
+    with pytest.raises(L.CatcocError, match="at most 2 k slices"):
+        ops.matmul_allreduce(a, b, [], 0, 1, split_k=4, workspace=torch.zeros(1 << 24, dtype=torch.uint8, device=DEV))
+    with pytest.raises(L.CatcocError, match="needs a workspace"):
+        ops.matmul_allreduce(a, b, [], 0, 1, split_k=2)
+    with pytest.raises(L.CatcocError, match="workspace too small"):
+        ops.matmul_allreduce(a, b, [], 0, 1, workspace=torch.zeros(4096, dtype=torch.uint8, device=DEV))
 
 
 @pytest.mark.parametrize("case", [(1, 512, 1024, 8, 0, 1, 0), (16, 512, 2048, 8, 0, 2, 0), (16, 384, 1024, 8, 6, 10, 4),
@@ -397,6 +440,53 @@ def test_allgather_matmul_reads_shards_in_place(dtype, shape):
     torch.cuda.synchronize()
     full = oracle.gemm_half_f32(np.concatenate(shards, 0), B, dtype)
     _check_float(host16(out), want, full, dtype, K)
+
+
+@pytest.mark.parametrize("dtype", [oracle.BF16, oracle.FP16])
+def test_float_few_tiles_k_sliced(dtype):
+    # two k slices per tile: an fp32 sum of two partials, the same whichever slice arrives last, so repeated
+    # launches agree bit for bit, and the result stays inside the float tolerance of the unsliced oracle
+    _need_gpu()
+    rng = np.random.default_rng(24)
+    tdt = TORCH_DT[dtype]
+    # all-gather: 8 shards of 128 rows, 32 tiles
+    ml, N, K, P, rank = 128, 512, 2048, 8, 3
+    shards = [_rand16(rng, (ml, K), dtype) for _ in range(P)]
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    want = oracle.allgather_matmul(shards, B, dtype)
+    need, f = ops.kslice_plan(L.ALLGATHER_MATMUL, tdt, ml, K, N, rank, P)
+    assert f == 2
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    dsh = [dev16(x, dtype) for x in shards]
+    outs = []
+    for _ in range(3):
+        out = ops.allgather_matmul(dsh[rank], [dsh[r] for r in range(P) if r != rank], dev16(B, dtype), rank, P, workspace=ws)
+        torch.cuda.synchronize()
+        outs.append(host16(out))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    _check_float(outs[0], want, oracle.gemm_half_f32(np.concatenate(shards, 0), B, dtype), dtype, K)
+    # reduce-scatter with peers and all-reduce, 16 tiles each
+    M, N, K, P, rank = 1024, 512, 1024, 4, 2
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    part, want = oracle.matmul_reduce(A, B, dtype, rank * rows, rows, peers, want_partial=True)
+    need, f = ops.kslice_plan(L.MATMUL_REDUCE_SCATTER, tdt, M, K, N, rank, P)
+    assert f == 2
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    out = ops.matmul_reduce_scatter(dev16(A, dtype), dev16(B, dtype), [dev(p) for p in peers], rank, P, acc_dump=dump, workspace=ws)
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part[rank * rows:(rank + 1) * rows] + sum(peers), dtype, K)
+    assert np.abs(dump.cpu().numpy() - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
+    fullp = [rng.standard_normal((M, N)).astype(np.float32)]
+    part, want = oracle.matmul_reduce(A, B, dtype, 0, M, fullp, want_partial=True)
+    need, f = ops.kslice_plan(L.MATMUL_ALLREDUCE, tdt, M, K, N, 0, 2)
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    out = ops.matmul_allreduce(dev16(A, dtype), dev16(B, dtype), [dev(fullp[0])], 0, 2, workspace=ws)
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part + fullp[0], dtype, K)
 
 
 def test_float_transposed_operands_general_kernel():
