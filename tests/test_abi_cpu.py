@@ -172,6 +172,16 @@ def test_splitk_launch_order_is_a_permutation_that_groups_b_readers(so):
 
 def test_workspace_size_queries(so):
     from mm_rs_with_catlass_amd import ops
+    import torch
+    # k slices of few-tile launches: fill the CUs once, at least eight k steps per slice, two slices at most for floats
+    assert ops.kslice_plan(L.ALLGATHER_MATMUL, torch.bfloat16, 512, 4096, 1024, 0, 8) == (128 * 2 * 131072 + 512, 2)
+    assert ops.kslice_plan(L.MATMUL_ALLREDUCE, torch.float16, 512, 1024, 1024, 0, 2) == (16 * 2 * 131072 + 256, 2)
+    assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 8192, 1792, 4096, 0, 8) == (0, 1)       # 1024 tiles
+    assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024, 4096, 1024, 0, 8) == (32 * 8 * 131072 + 256, 8)
+    assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024, 4096, 1024, 0, 8, split_k=2)[1] == 2
+    assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024 + 8, 4096, 1024, 0, 8) == (0, 1)   # ragged rows
+    with pytest.raises(L.CatcocError, match="at most 2 k slices"):
+        ops.kslice_plan(L.MATMUL_ALLREDUCE, torch.float16, 512, 1024, 1024, 0, 2, split_k=4)
     need, f, tiles = ops.splitk_plan(16, 8192, 8192, 8, 0, 2)
     assert (f, tiles) == (oracle.splitk_factor(16, 8192, 8192, 256, 128, 128, 256), 64)
     assert need == f * tiles * 128 * 128 * 4 + 256
