@@ -286,6 +286,11 @@ CATCOC_API int catcoc_task_tile(int commType, const CocTilingParams *tiling, con
  * simply runs tasks i, i + BLOCK_NUM, ... (quant_matmul_reduce_scatter.hpp:166-170). */
 CATCOC_API uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
                                        uint32_t wg);
+/* The same with the tile: what workgroup `wg` of the launch computes, exactly as the kernel works it out (the
+ * large-tile kernels take a division-free route through constants prepared per launch; this entry point is how
+ * tests compare that route with catcoc_launch_task + catcoc_task_tile).  Returns 0 past the end of the launch. */
+CATCOC_API int catcoc_launch_tile(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t wg,
+                                  uint32_t *task, uint32_t *targetRank, uint32_t *row, uint32_t *col, uint32_t *wsRow);
 /* The task workgroup `wg` of a launch with `tasks` tasks runs (XCD-aware chunking unless
  * CATCOC_FLAG_LINEAR_ORDER); a bijection on [0,tasks). */
 CATCOC_API uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags);

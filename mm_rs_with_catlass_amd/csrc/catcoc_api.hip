@@ -549,6 +549,37 @@ int catcoc_task_tile(int commType, const CocTilingParams *tiling, const CatcocSy
     return 1;
 }
 
+int catcoc_launch_tile(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t wg, uint32_t *task,
+                       uint32_t *targetRank, uint32_t *row, uint32_t *col, uint32_t *wsRow)
+{
+    Plan p;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
+    d = *desc;
+    d.flags &= ~CATCOC_OUTBOUND_MASK;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    const int dataType = commType == QUANT_MATMUL_REDUCE_SCATTER ? INT8 : FP16;
+    if (make_plan(commType, dataType, tiling, &d, 0, 0, p)) return 0;
+    ok();
+    const SchedParams &s = p.args.sched;
+    const bool linear = (p.args.flags & GF_LINEAR_ORDER) != 0;
+    uint32_t t;
+    TileInfo ti;
+    if (p.dma) {
+        if (!launch_tile(s, wg, linear, p.args.keptRank, t, ti)) return 0;
+    } else {
+        if (wg >= s.coreLoops) return 0;
+        t = launch_order_task(s, wg, linear, p.args.keptRank);
+        if (!task_tile(s, t, ti)) return 0;
+    }
+    if (task) *task = t;
+    if (targetRank) *targetRank = ti.targetRank;
+    if (row) *row = ti.row;
+    if (col) *col = ti.col;
+    if (wsRow) *wsRow = ti.wsRow;
+    return 1;
+}
+
 uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t wg)
 {
     Plan p;

@@ -117,9 +117,9 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             pos = blockIdx.x / kSlices;
         }
     }
-    const uint32_t task = launch_task(sp, pos, linear, args.keptRank);
+    uint32_t task;
     TileInfo ti;
-    if (!task_tile(sp, task, ti)) return;
+    if (!launch_tile(sp, pos, linear, args.keptRank, task, ti)) return;
     // The kept tiles are the longest chain of a reduce-scatter launch (main loop, then the peers' partials):
     // their waves get priority over the other workgroup on the CU so that the chain starts its streaming early.
     if (sp.op == OP_REDUCE_SCATTER && sp.P > 1 && ti.row >= args.keptBegin && ti.row < args.keptBegin + args.keptRows)
@@ -132,10 +132,13 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const unsigned char *Bg = (const unsigned char *)args.b + (size_t)ti.col * ES;
     // k steps (64 bytes of K each) of this workgroup: all of them, or its slice
     const uint32_t nkAll = args.K * ES / 64;
-    const uint32_t kFirst = (uint32_t)(((uint64_t)nkAll * slice) / kSlices);
-    const uint32_t nk = (uint32_t)(((uint64_t)nkAll * (slice + 1u)) / kSlices) - kFirst;
-    Ag += (size_t)kFirst * 64;
-    Bg += (size_t)kFirst * (64 / ES) * ldbB;
+    uint32_t nk = nkAll;
+    if (kSlices > 1) {   // (at most 16 slices of fewer than 2^24 steps: 32-bit products)
+        const uint32_t kFirst = nkAll * slice / kSlices;
+        nk = nkAll * (slice + 1u) / kSlices - kFirst;
+        Ag += (size_t)kFirst * 64;
+        Bg += (size_t)kFirst * (64 / ES) * ldbB;
+    }
 
     // ---- copy descriptors ---------------------------------------------------
     // Every copy a wave issues has its own global pointer, advanced after each issue, and a scalar LDS address:

@@ -16,6 +16,28 @@ namespace catcoc {
 CATCOC_HD uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1u) / b; }
 CATCOC_HD uint32_t umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
 
+// Division by a launch constant without the float round trip a 32-bit division compiles to on the GPU (every
+// workgroup runs a few dozen of them before its first load).  m = floor(2^32 / d); the estimate mulhi(n, m) is at
+// most two short of n / d for any 32-bit n, so two conditional corrections make it exact.
+struct FastDiv { uint32_t d, m; };
+CATCOC_HD FastDiv make_fast_div(uint32_t d)
+{
+    FastDiv f;
+    f.d = d ? d : 1u;
+    const uint64_t m = 0x100000000ull / f.d;
+    f.m = m > 0xffffffffull ? 0xffffffffu : (uint32_t)m;
+    return f;
+}
+CATCOC_HD uint32_t fast_div(uint32_t n, const FastDiv &f, uint32_t &rem)
+{
+    uint32_t q = (uint32_t)(((uint64_t)n * f.m) >> 32);
+    uint32_t r = n - q * f.d;
+    if (r >= f.d) { ++q; r -= f.d; }
+    if (r >= f.d) { ++q; r -= f.d; }
+    rem = r;
+    return q;
+}
+
 // Walk a 2-D grid in bands of `width` lines along the banded axis: inside a band
 // the banded axis runs fastest; with `serpentine` the other axis runs backwards
 // on odd bands.  The last band may be narrower.
@@ -154,6 +176,13 @@ struct SchedParams {
     uint32_t commInterval;
     uint32_t stages;
     uint32_t off, dir;
+    // XCD-block launch order worked out once per launch (xcd_launch_tile): the cut of the tile grid and the
+    // divisors of the workgroup -> tile arithmetic
+    uint32_t xOk;                 // the order applies to this launch
+    uint32_t xRxLog, xCxLog;      // row parts x column parts = 8, as powers of two
+    uint32_t xRowsPer, xColsPer;  // tile rows / tile columns of one XCD's block
+    uint32_t xPerRank, xCommLoops, xLastPerRank;   // tasks of one rank in a full round; rounds; the same in the last round
+    FastDiv dColsPer, dLoopsM, dBand, dPerRank, dStages, dBpc;
 };
 
 struct TileInfo {
@@ -164,6 +193,8 @@ struct TileInfo {
     uint32_t rowsValid, colsValid;
     uint32_t wsRow;       // first row of the tile in the reference's tile-linear workspace
 };
+
+CATCOC_HD void fill_xcd_order(SchedParams &s);
 
 CATCOC_HD SchedParams make_sched(uint32_t op, uint32_t M, uint32_t N, uint32_t P, uint32_t m0, uint32_t n0,
                                  uint32_t blockNum, uint32_t commInterval, uint32_t stages, uint32_t off,
@@ -184,6 +215,7 @@ CATCOC_HD SchedParams make_sched(uint32_t op, uint32_t M, uint32_t N, uint32_t P
     s.stages = stages;
     s.off = off;
     s.dir = dir;
+    fill_xcd_order(s);
     return s;
 }
 
@@ -333,6 +365,85 @@ CATCOC_HD bool xcd_block_task(const SchedParams &s, uint32_t keptRank, uint32_t 
     return true;
 }
 
+// The launch constants of the XCD-block order (part of SchedParams, filled by make_sched).
+CATCOC_HD void fill_xcd_order(SchedParams &s)
+{
+    XcdBlock g;
+    s.xOk = (s.stages != 0 && s.blockPerComm != 0 && s.blockPerComm % (s.op == OP_REDUCE_SCATTER ? s.P : 1u) == 0 &&
+             xcd_block(s, 0, 0, g)) ? 1u : 0u;
+    s.xRxLog = s.xCxLog = s.xRowsPer = s.xColsPer = s.xPerRank = s.xCommLoops = s.xLastPerRank = 0;
+    s.dColsPer = s.dLoopsM = s.dBand = s.dPerRank = s.dStages = s.dBpc = make_fast_div(1);
+    if (!s.xOk) return;
+    while ((1u << s.xRxLog) < g.RX) ++s.xRxLog;
+    s.xCxLog = 3u - s.xRxLog;
+    s.xRowsPer = g.rowsPer;
+    s.xColsPer = g.colsPer;
+    const uint32_t ranks = s.op == OP_REDUCE_SCATTER ? s.P : 1u;
+    s.xPerRank = s.blockPerComm / ranks;
+    s.xCommLoops = ceil_div(s.coreLoops, s.blockPerComm);
+    s.xLastPerRank = (s.coreLoops - (s.xCommLoops - 1u) * s.blockPerComm) / ranks;
+    s.dColsPer = make_fast_div(g.colsPer);
+    s.dLoopsM = make_fast_div(s.loopsM);
+    s.dBand = make_fast_div(s.off);
+    s.dPerRank = make_fast_div(s.xPerRank);
+    s.dStages = make_fast_div(s.stages);
+    s.dBpc = make_fast_div(s.blockPerComm);
+}
+
+// xcd_block_task followed by task_tile, from the launch constants and without a division: workgroup -> task and tile.
+// Only for launches with s.xOk.
+CATCOC_HD void xcd_launch_tile(const SchedParams &s, uint32_t keptRank, uint32_t wg, uint32_t &task, TileInfo &ti)
+{
+    const bool rs = s.op == OP_REDUCE_SCATTER;
+    const uint32_t x = wg & 7u, j = wg >> 3;
+    const uint32_t rp = x >> s.xCxLog, cp = x - (rp << s.xCxLog);
+    uint32_t i0 = 0, i1 = 0;
+    if (rs && s.P > 1) {
+        const uint32_t lo = keptRank * s.loopsM, hi = lo + s.loopsM, up = (1u << s.xRxLog) - 1u;
+        i0 = umin(lo > rp ? (lo - rp + up) >> s.xRxLog : 0u, s.xRowsPer);
+        i1 = umin(hi > rp ? (hi - rp + up) >> s.xRxLog : 0u, s.xRowsPer);
+    }
+    uint32_t ci;
+    const uint32_t ri = fast_div(j, s.dColsPer, ci);
+    const uint32_t nk = i1 - i0;
+    uint32_t i;
+    if (ri < nk) i = i0 + ri;
+    else { const uint32_t t = ri - nk; i = t < i0 ? t : t + nk; }
+    const uint32_t gr = rp + (i << s.xRxLog), nIdx = cp * s.xColsPer + ci;
+    uint32_t mIdx;
+    const uint32_t rank = fast_div(gr, s.dLoopsM, mIdx);
+    // position of (mIdx, nIdx) in the swizzled order of one rank's grid (banded_index with the band width s.off)
+    const uint32_t posBanded = s.dir == 0 ? mIdx : nIdx, posOther = s.dir == 0 ? nIdx : mIdx;
+    const uint32_t lenBanded = s.dir == 0 ? s.loopsM : s.loopsN, lenOther = s.dir == 0 ? s.loopsN : s.loopsM;
+    uint32_t inBand;
+    const uint32_t band = fast_div(posBanded, s.dBand, inBand);
+    const uint32_t w = umin(s.off, lenBanded - band * s.off);
+    const uint32_t q = (band & 1u) ? lenOther - 1u - posOther : posOther;
+    const uint32_t inRank = band * s.off * lenOther + q * w + inBand;
+    uint32_t round, b;
+    if (rs) {
+        uint32_t idx;
+        round = fast_div(inRank, s.dPerRank, idx);
+        b = rank * (round == s.xCommLoops - 1u ? s.xLastPerRank : s.xPerRank) + idx;
+        task = round * s.blockPerComm + b;
+    } else {
+        task = inRank;
+        round = fast_div(task, s.dBpc, b);
+    }
+    uint32_t stage;
+    fast_div(round, s.dStages, stage);
+    ti.targetRank = rank;
+    ti.rowInRank = mIdx * s.m0;
+    ti.row = rank * s.mRank + ti.rowInRank;
+    ti.col = nIdx * s.n0;
+    ti.rowsValid = umin(s.m0, s.mRank - ti.rowInRank);
+    ti.colsValid = umin(s.n0, s.N - ti.col);
+    ti.wsRow = (stage * s.blockPerComm + b) * s.m0;
+}
+
+// Workgroup -> task and tile of a launch of the direct-to-LDS kernels; false past the end of the launch.
+CATCOC_HD bool launch_tile(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank, uint32_t &task, TileInfo &ti);
+
 // Workgroup -> task of a launch: the XCD-block order where it applies, else XCD-aware chunking with the kept
 // rank's tiles first.  Either way the kept tiles are among the first ceil(kept / 128) * 128 workgroups.
 CATCOC_HD uint32_t launch_task(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank)
@@ -341,6 +452,17 @@ CATCOC_HD uint32_t launch_task(const SchedParams &s, uint32_t wg, bool linear, u
     uint32_t task;
     if (xcd_block_task(s, keptRank, wg, task)) return task;
     return kept_first_task(s, keptRank, workgroup_task(wg, s.coreLoops, false));
+}
+
+CATCOC_HD bool launch_tile(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank, uint32_t &task, TileInfo &ti)
+{
+    if (wg >= s.coreLoops) return false;
+    if (!linear && s.xOk) {
+        xcd_launch_tile(s, keptRank, wg, task, ti);
+        return true;
+    }
+    task = launch_task(s, wg, linear, keptRank);
+    return task_tile(s, task, ti);
 }
 
 // Workgroup -> task of a launch: XCD-aware chunking, then kept-first ordering.

@@ -64,7 +64,7 @@ EXPORTS = [
     "catcoc_get_task_count", "catcoc_get_tilings", "catcoc_check_comm_interval_reduce_scatter",
     "catcoc_check_comm_interval_allreduce", "catcoc_check_comm_interval_allgather", "catcoc_get_splitk_factor",
     "catcoc_default_tiling", "catcoc_swizzle_block_coord", "catcoc_splitk_block_coord", "catcoc_splitk_actual_k", "catcoc_splitk_launch_task",
-    "catcoc_allgather_block_coord", "catcoc_comm_block_idx", "catcoc_task_tile", "catcoc_workgroup_task", "catcoc_launch_task",
+    "catcoc_allgather_block_coord", "catcoc_comm_block_idx", "catcoc_task_tile", "catcoc_workgroup_task", "catcoc_launch_task", "catcoc_launch_tile",
     "catcoc_device_info", "catcoc_version",
 ]
 
@@ -152,6 +152,8 @@ def load():
     L.catcoc_comm_block_idx.argtypes = [u32] * 6 + [pu, pu]
     L.catcoc_task_tile.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32] + [pu] * 4
     L.catcoc_task_tile.restype = C.c_int
+    L.catcoc_launch_tile.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32] + [pu] * 5
+    L.catcoc_launch_tile.restype = C.c_int
     L.catcoc_workgroup_task.argtypes = [u32, u32, u32]
     L.catcoc_workgroup_task.restype = u32
     L.catcoc_device_info.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_char_p, C.c_int]

@@ -4,6 +4,7 @@ import ctypes as C
 import re
 import os
 
+import numpy as np
 import pytest
 
 import oracle
@@ -147,6 +148,53 @@ def test_launch_order_is_a_bijection_with_kept_tiles_first_or_last(so):
             # 128 workgroups that the XCD-aware orders apply
             span = -(-nk // 128) * 128
             assert max(wg for wg in range(n) if kept[wg]) < span
+
+
+def test_launch_tile_equals_launch_task_then_task_tile(so):
+    # the kernels work out workgroup -> task and tile through per-launch constants and reciprocal multiplies; the
+    # result has to be what the plain integer route gives, for every workgroup, operator, swizzle and round layout
+    from mm_rs_with_catlass_amd import ops
+    cases = [(L.QUANT_MATMUL_REDUCE_SCATTER, 8192, 1792, 4096, 8, 0, 128, {}),
+             (L.QUANT_MATMUL_REDUCE_SCATTER, 8192, 1792, 4096, 8, 5, 256, {}),
+             (L.QUANT_MATMUL_REDUCE_SCATTER, 4096, 512, 2048, 4, 3, 128, dict(block_num=20, stages=3, swizzle=(3, 0))),
+             (L.QUANT_MATMUL_REDUCE_SCATTER, 6144, 256, 1280, 2, 1, 128, dict(block_num=6, swizzle=(5, 1))),
+             (L.QUANT_MATMUL_REDUCE_SCATTER, 2048, 256, 1024, 1, 0, 128, {}),
+             (L.MATMUL_REDUCE_SCATTER, 4096, 1792, 4096, 8, 7, 128, {}),
+             (L.MATMUL_ALLREDUCE, 2048, 1024, 2048, 2, 0, 128, dict(block_num=20, stages=2, swizzle=(2, 1))),
+             (L.MATMUL_ALLREDUCE, 512, 1024, 1024, 2, 1, 128, {}),
+             (L.ALLGATHER_MATMUL, 512, 4096, 1024, 8, 2, 128, {})]
+    task, tr, row, col, wsr = (u32() for _ in range(5))
+    tr2, row2, col2, wsr2 = (u32() for _ in range(4))
+    for comm, M, K, N, P, rank, m0, kw in cases:
+        t = ops.default_tiling(M, K, N, P, m0=m0, n0=256, k0=256)
+        d = L.make_desc(rank, P, **kw)
+        n = so.catcoc_get_task_count(comm, C.byref(t), C.byref(d))
+        assert n > 0, L.last_error()
+        seen = set()
+        for wg in range(n):
+            assert so.catcoc_launch_tile(comm, C.byref(t), C.byref(d), wg, C.byref(task), C.byref(tr), C.byref(row), C.byref(col), C.byref(wsr)) == 1
+            assert task.value == so.catcoc_launch_task(comm, C.byref(t), C.byref(d), wg), (comm, M, N, P, wg)
+            assert so.catcoc_task_tile(comm, C.byref(t), C.byref(d), task.value, C.byref(tr2), C.byref(row2), C.byref(col2), C.byref(wsr2)) == 1
+            assert (tr.value, row.value, col.value, wsr.value) == (tr2.value, row2.value, col2.value, wsr2.value), (comm, M, N, P, wg)
+            seen.add(task.value)
+        assert len(seen) == n
+        assert so.catcoc_launch_tile(comm, C.byref(t), C.byref(d), n, None, None, None, None, None) == 0
+
+
+def test_reciprocal_division_is_exact():
+    # the formula of the schedulers' FastDiv (m = floor(2^32 / d), estimate mulhi(n, m), two corrections)
+    rng = np.random.default_rng(3)
+    ds = np.concatenate([np.arange(1, 300), rng.integers(1, 2 ** 32, 300), [2 ** 31, 2 ** 32 - 1, 65535, 65536, 65537]]).astype(np.uint64)
+    ns = np.concatenate([np.arange(0, 300), rng.integers(0, 2 ** 32, 500), [2 ** 32 - 1, 2 ** 31, 2 ** 31 - 1]]).astype(np.uint64)
+    for d in ds:
+        m = min((1 << 32) // int(d), 0xffffffff)
+        q = (ns * np.uint64(m)) >> np.uint64(32)
+        r = ns - q * d
+        for _ in range(2):
+            up = r >= d
+            q = q + up
+            r = r - up * d
+        assert np.array_equal(q, ns // d) and np.array_equal(r, ns % d), int(d)
 
 
 def test_splitk_launch_order_is_a_permutation_that_groups_b_readers(so):
