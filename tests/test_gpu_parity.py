@@ -194,6 +194,24 @@ def test_quant_rs_few_tiles_k_sliced(case):
             assert cs[task] == blk.sum(), task
 
 
+def test_quant_rs_few_tiles_k_sliced_outbound_store():
+    # the sliced launch with the other ranks' tiles stored (not just summed): the last slice writes the fp32 tile
+    M, N, K, P, rank = 1024, 512, 2048, 4, 2
+    r = quant_case(np.random.default_rng(77), M, N, K, P, rank, bias=True, outbound=True, launches=2, kslices=(0, 4))
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    import ctypes as C
+    tr, row, col, wsr = (C.c_uint32() for _ in range(4))
+    ob = r["outbound"].cpu().numpy().reshape(-1, 256)
+    deq = oracle.dequant(r["acc"], r["s2"], r["s1"])
+    for task in range(r["ntasks"]):
+        L.load().catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row), C.byref(col), C.byref(wsr))
+        if tr.value == rank:
+            continue
+        want = deq[row.value:row.value + 128, col.value:col.value + 256]
+        assert np.array_equal(ob[wsr.value:wsr.value + 128].view(np.uint32), want.view(np.uint32)), task
+
+
 def test_k_slice_rejections():
     _need_gpu()
     a = torch.zeros((512, 1024), dtype=torch.float16, device=DEV)
@@ -208,7 +226,8 @@ def test_k_slice_rejections():
 
 @pytest.mark.parametrize("case", [(1, 512, 1024, 8, 0, 1, 0), (16, 512, 2048, 8, 0, 2, 0), (16, 384, 1024, 8, 6, 10, 4),
                                   (64, 256, 4096, 8, 8, 8, 0), (128, 640, 2048, 8, 112, 16, 0), (200, 256, 1088, 4, 100, 50, 3),
-                                  (33, 128, 64, 2, 0, 33, 0), (512, 1024, 1024, 8, 0, 64, 2)])
+                                  (33, 128, 64, 2, 0, 33, 0), (512, 1024, 1024, 8, 0, 64, 2), (64, 256, 2048, 4, 0, 16, 8),
+                                  (48, 384, 1536, 1, 0, 48, 6), (256, 256, 320, 2, 128, 128, 0)])
 def test_quant_skinny_m_splitk(case):
     # decode shapes: any m, explicit kept rows, k slices meet through the workspace; int32 sums are exact
     _need_gpu()
