@@ -119,7 +119,9 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     plan.edge = !(mRank % m0 == 0 && t->n % n0 == 0 && t->k % (64 / es) == 0);
     plan.dtype = dt;
     plan.blockNum = blockNum;
-    plan.dma = fastShape && !plan.edge && (m0 == 128 || m0 == 256) && !transA && !transB && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
+    // (B as [n,k] runs the 128-row direct-to-LDS kernel when its rows of k are 16-byte multiples)
+    plan.dma = fastShape && !plan.edge && (m0 == 256 || (m0 == 128 && (!transB || ((uint64_t)t->k * es) % 16 == 0))) && !transA &&
+               (m0 == 128 || !transB) && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
 
     GemmArgs &a = plan.args;
     memset(&a, 0, sizeof(a));

@@ -74,7 +74,9 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 // Geometries (every wave computes 64 x 128: MB = 2 row blocks of 32, 4 column blocks of 32; two wave columns):
 //   WM 2 -> 128x256 tile, 4 waves, 3 stages (72 KiB LDS, two workgroups per CU);
 //   WM 4 -> 256x256 tile, 8 waves (128 KiB LDS, one workgroup per CU): half the L2 -> LDS traffic per MAC.
-template <uint32_t DT, int WM>
+//   TB   -> B is given as [n][k] (k contiguous, the layout of a weight matrix stored output-major): its tiles are then
+//           staged and read exactly like A's, rows of 64 bytes of k, and need no transposing LDS reads.
+template <uint32_t DT, int WM, bool TB = false>
 __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
 {
     static_assert(WM == 2 || WM == 4, "supported geometries");
@@ -129,7 +131,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const bool gather = sp.op == OP_ALLGATHER;
     const unsigned char *Ag = (const unsigned char *)args.a[gather ? ti.targetRank : 0] +
                               (int64_t)(gather ? ti.rowInRank : ti.row) * ldaB;
-    const unsigned char *Bg = (const unsigned char *)args.b + (size_t)ti.col * ES;
+    const unsigned char *Bg = (const unsigned char *)args.b + (TB ? (size_t)ti.col * ldbB : (size_t)ti.col * ES);
     // k steps (64 bytes of K each) of this workgroup: all of them, or its slice
     const uint32_t nkAll = args.K * ES / 64;
     uint32_t nk = nkAll;
@@ -137,7 +139,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         const uint32_t kFirst = nkAll * slice / kSlices;
         nk = nkAll * (slice + 1u) / kSlices - kFirst;
         Ag += (size_t)kFirst * 64;
-        Bg += (size_t)kFirst * (64 / ES) * ldbB;
+        Bg += TB ? (size_t)kFirst * 64 : (size_t)kFirst * (64 / ES) * ldbB;
     }
 
     // ---- copy descriptors ---------------------------------------------------
@@ -160,10 +162,13 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     // B, 1-byte elements: copy j covers k rows 4j..4j+3; lane -> row 4j + lane/16, LDS slot lane&15 holds column
     // chunk slot^((row&7)<<1).  2-byte elements (32 k rows x 512 bytes): copy j covers k rows 2j, 2j+1; lane -> row
     // 2j + lane/32, slot lane&31 holds chunk slot^((row&3)<<2).
+    // B given as [n][k]: copy j covers tile columns 16j..16j+15, one 64-byte row of k each, laid out like A.
     const unsigned char *gB[B_DMA];
 #pragma unroll
     for (int jj = 0; jj < B_DMA; ++jj) {
-        if constexpr (ES == 1) {
+        if constexpr (TB) {
+            gB[jj] = Bg + (size_t)(16 * (w + NW * jj) + (lane >> 2)) * ldbB + (((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+        } else if constexpr (ES == 1) {
             const int row = 4 * (w + NW * jj) + (lane >> 4);
             gB[jj] = Bg + (size_t)row * ldbB + (((lane & 15) ^ ((row & 7) << 1)) * 16);
         } else {
@@ -171,7 +176,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             gB[jj] = Bg + (size_t)row * ldbB + (((lane & 31) ^ ((row & 3) << 2)) * 16);
         }
     }
-    const size_t bStep = (size_t)(64 / ES) * ldbB;
+    const size_t bStep = TB ? (size_t)64 : (size_t)(64 / ES) * ldbB;
     auto issue_b = [&](uint32_t ldsStage) {   // next k step of B
 #pragma unroll
         for (int jj = 0; jj < B_DMA; ++jj) {
@@ -211,7 +216,12 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     }
     constexpr int B_KK = (ES == 1) ? 32 * 256 : 16 * 512;     // bytes of a stage per 32-byte k slab
     constexpr int B_HALF = (ES == 1) ? 8 * 256 : 4 * 512;     // second transpose read of a fragment
+    const uint32_t bt_lds = (wn * 128 + c32) * 64, bt_sw = (c32 >> 2) & 3;   // [n][k] stage: row of column c32, chunk swizzle
     auto read_b1 = [&](v4i (&bf)[4], const unsigned char *sb, int kk, int nb) {
+        if constexpr (TB) {
+            bf[nb] = *(const v4i *)(sb + bt_lds + nb * 32 * 64 + (((2 * kk + h) ^ bt_sw) * 16));
+            return;
+        }
         const unsigned char *p = sb + b_lds[nb] + kk * B_KK;
         v2i t0, t1;
         if constexpr (ES == 1) {

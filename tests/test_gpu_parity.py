@@ -132,6 +132,16 @@ def test_quant_rs_transposed_b():
     quant_case(np.random.default_rng(3), 1024, 512, 256, 8, 2, trans_b=True)
 
 
+@pytest.mark.parametrize("case", [(4096, 1024, 1792, 8, 3, None), (2048, 2048, 320, 2, 1, None), (1024, 1024, 2048, 4, 1, (0, 4)),
+                                  (1024, 512, 1024, 2, 0, (3, 3))])
+def test_quant_rs_weights_stored_n_by_k(case):
+    # B given as [n,k] (the usual layout of a weight matrix): full tiles run the direct-to-LDS kernel, which then
+    # stages B like A and needs no transposing reads; also cut into k slices; everything stays bit-exact
+    M, N, K, P, rank, ks = case
+    r = quant_case(np.random.default_rng(80 + rank), M, N, K, P, rank, bias=True, trans_b=True, launches=2, kslices=ks)
+    assert r["exact"] == r["total"]
+
+
 @pytest.mark.parametrize("shape", [(800, 260, 208), (8 * 130, 516, 80), (64, 256, 16), (8, 4, 16)])
 def test_quant_rs_ragged_edges(shape):
     M, N, K = shape
@@ -506,6 +516,42 @@ def test_float_few_tiles_k_sliced(dtype):
     out = ops.matmul_allreduce(dev16(A, dtype), dev16(B, dtype), [dev(fullp[0])], 0, 2, workspace=ws)
     torch.cuda.synchronize()
     _check_float(host16(out), want, part + fullp[0], dtype, K)
+
+
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+def test_float_weights_stored_n_by_k(dtype):
+    _need_gpu()
+    rng = np.random.default_rng(25)
+    tdt = TORCH_DT[dtype]
+    M, N, K, P, rank = 1024, 768, 640, 4, 3
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    Bt = np.ascontiguousarray(B.T)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    part, want = oracle.matmul_reduce(A, B, dtype, rank * rows, rows, peers, want_partial=True)
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    out = ops.matmul_reduce_scatter(dev16(A, dtype), dev16(Bt, dtype), [dev(p) for p in peers], rank, P, trans_b=True, acc_dump=dump)
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part[rank * rows:(rank + 1) * rows] + sum(peers), dtype, K)
+    assert np.abs(dump.cpu().numpy() - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
+    # the same operands through the row-major path: same MFMAs in the same k order, so the fp32 partials are identical
+    dump2 = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    ops.matmul_reduce_scatter(dev16(A, dtype), dev16(B, dtype), [dev(p) for p in peers], rank, P, acc_dump=dump2)
+    torch.cuda.synchronize()
+    assert torch.equal(dump, dump2)
+    # all-gather with [n,k] weights and two k slices
+    ml, N, K, P, rank = 128, 512, 2048, 8, 6
+    shards = [_rand16(rng, (ml, K), dtype) for _ in range(P)]
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    want = oracle.allgather_matmul(shards, B, dtype)
+    need, f = ops.kslice_plan(L.ALLGATHER_MATMUL, tdt, ml, K, N, rank, P)
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    dsh = [dev16(x, dtype) for x in shards]
+    out = ops.allgather_matmul(dsh[rank], [dsh[r] for r in range(P) if r != rank], dev16(np.ascontiguousarray(B.T), dtype), rank, P,
+                               trans_b=True, workspace=ws)
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, oracle.gemm_half_f32(np.concatenate(shards, 0), B, dtype), dtype, K)
 
 
 def test_float_transposed_operands_general_kernel():
