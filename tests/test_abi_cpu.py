@@ -317,3 +317,11 @@ def test_rejected_launch_launches_nothing_and_reports(so):
         L.check()
     so.catcoc_quant_matmul_reduce_scatter(None, 0, 16, 16, 16, 16, None, None, 16, None, 1024, 512, 256)
     assert so.catcoc_last_status() != 0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout == ""
