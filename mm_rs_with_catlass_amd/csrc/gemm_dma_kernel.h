@@ -119,9 +119,17 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             pos = blockIdx.x / kSlices;
         }
     }
+    if (pos >= sp.coreLoops) return;
     uint32_t task;
     TileInfo ti;
-    if (!launch_tile(sp, pos, linear, args.keptRank, task, ti)) return;
+    if (!linear && sp.xOk) {
+        xcd_launch_tile(sp, args.keptRank, pos, task, ti);
+    } else {
+        task = launch_task(sp, pos, linear, args.keptRank);
+        TileInfo tg;   // (a separate object: filled in place, the tile of both routes ends up in memory instead of registers)
+        task_tile(sp, task, tg);
+        ti = tg;
+    }
     // The kept tiles are the longest chain of a reduce-scatter launch (main loop, then the peers' partials):
     // their waves get priority over the other workgroup on the CU so that the chain starts its streaming early.
     if (sp.op == OP_REDUCE_SCATTER && sp.P > 1 && ti.row >= args.keptBegin && ti.row < args.keptBegin + args.keptRows)
