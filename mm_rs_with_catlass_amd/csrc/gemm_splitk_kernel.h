@@ -303,65 +303,67 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     }
 
     // ---- epilogue on the rows that exist -----------------------------------------------
-    // Per 32-row block: bias, dumps, checksum of the rows that are not kept; then, for the register slots that
-    // hold kept rows only, dequant, the peers in slot order (the first block with kept rows has its first eight
-    // peers in registers already; anything else is fetched eight peers at a time in one round trip) and the
-    // 16-bit store.
+    // First a cheap pass over every 32-row block: bias, dumps, checksum of the rows that are not kept.  Then ONE loop
+    // body, run once per block with kept rows (a run-time loop: this code executes once per tile, and unrolled per
+    // block it was several times the size of the instruction cache): the block's registers are selected, dequantised,
+    // the peers added in slot order eight at a time (the first block's first eight are in registers already, the
+    // others are fetched into the same registers in one round trip) and the 16-bit rows stored.
     long long csum = 0;
 #pragma unroll
     for (int mb = 0; mb < MBW; ++mb) {
         if ((uint32_t)mb * 32 >= rowsValid) break;
         const KeptRows k = kept_rows(mb);
         const uint32_t vrel = mb * 32 + 4u * h;   // slot r is a row of A when slot_row(r) + vrel < rowsValid
-        int iv[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) iv[r] = acc[mb][r] + bv;
+        for (int r = 0; r < 16; ++r) acc[mb][r] += bv;
         if (args.checksum != nullptr) {   // rows that are not kept are only summed, and only on request
 #pragma unroll
-            for (int r = 0; r < 16; ++r) csum += (slot_row(r) + vrel < rowsValid && !lane_kept(k, r)) ? iv[r] : 0;
+            for (int r = 0; r < 16; ++r) csum += (slot_row(r) + vrel < rowsValid && !lane_kept(k, r)) ? acc[mb][r] : 0;
         }
         if (args.accDump) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                if (slot_row(r) + vrel < rowsValid) ((int32_t *)args.accDump)[(size_t)(row0 + vrel + slot_row(r)) * N + gcol] = iv[r];
+                if (slot_row(r) + vrel < rowsValid) ((int32_t *)args.accDump)[(size_t)(row0 + vrel + slot_row(r)) * N + gcol] = acc[mb][r];
         }
-        if (k.n == 0) continue;
-        if (args.cAccum) {
+        if (k.n != 0 && args.cAccum) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                if (lane_kept(k, r)) args.cAccum[(size_t)(row0 + vrel + slot_row(r) - args.keptBegin) * N + gcol] = iv[r];
+                if (lane_kept(k, r)) args.cAccum[(size_t)(row0 + vrel + slot_row(r) - args.keptBegin) * N + gcol] = acc[mb][r];
         }
+    }
+#pragma nounroll
+    for (uint32_t t = mbK; t < (uint32_t)MBW; ++t) {
+        const KeptRows k = kept_rows(t);
+        if (k.n == 0) continue;
+        // this block's accumulators and per-token scale, picked with uniform selects
+        int iv[16];
+        float sMt = sMrow[0];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) iv[r] = acc[0][r];
+#pragma unroll
+        for (int mb = 1; mb < MBW; ++mb)
+            if (t == (uint32_t)mb) {
+                sMt = sMrow[mb];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) iv[r] = acc[mb][r];
+            }
         float v[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-            v[r] = slot_active(k, r) ? __fmul_rn(__fmul_rn((float)iv[r], sN), __shfl(sMrow[mb], slot_row(r) + 4 * h, 64)) : 0.0f;
-        uint32_t p0 = 0;
-        if ((uint32_t)mb == mbK) {
+        for (int r = 0; r < 16; ++r) v[r] = __fmul_rn(__fmul_rn((float)iv[r], sN), __shfl(sMt, slot_row(r) + 4 * h, 64));
+        for (uint32_t p0 = 0; p0 < args.nPeers; p0 += 8) {
+            if (t != mbK || p0 != 0) fetch_peers(k, p0, pv0);
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                if (slot_active(k, r)) {
+            for (int q = 0; q < 8; ++q)
+                if (p0 + q < args.nPeers) {
 #pragma unroll
-                    for (int q = 0; q < 8; ++q)
-                        if ((uint32_t)q < args.nPeers) v[r] = __fadd_rn(v[r], pv0[q][r]);
-                }
-            p0 = 8;
-        }
-        for (; p0 < args.nPeers; p0 += 8) {
-            float pv[8][16];
-            fetch_peers(k, p0, pv);
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                if (slot_active(k, r)) {
-#pragma unroll
-                    for (int q = 0; q < 8; ++q)
-                        if (p0 + q < args.nPeers) v[r] = __fadd_rn(v[r], pv[q][r]);
+                    for (int r = 0; r < 16; ++r) v[r] = __fadd_rn(v[r], pv0[q][r]);
                 }
         }
         // signed: the block may start above the first kept row (only kept lanes dereference)
-        unsigned short *drow = (unsigned short *)args.d + ((int64_t)(row0 + vrel) - (int64_t)args.keptBegin) * args.ldd + gcol;
+        unsigned short *drow = (unsigned short *)args.d + ((int64_t)(row0 + t * 32 + 4u * h) - (int64_t)args.keptBegin) * args.ldd + gcol;
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-            if (slot_active(k, r) && lane_kept(k, r)) drow[(int64_t)slot_row(r) * args.ldd] = (unsigned short)f32_to_out16(v[r], args.outDtype);
+            if (lane_kept(k, r)) drow[(int64_t)slot_row(r) * args.ldd] = (unsigned short)f32_to_out16(v[r], args.outDtype);
     }
     if (args.checksum != nullptr) {
         long long *red = (long long *)smem + 8;
