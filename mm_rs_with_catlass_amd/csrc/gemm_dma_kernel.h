@@ -104,6 +104,14 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const int c32 = lane & 31, h = lane >> 5;
 
     const SchedParams &sp = args.sched;
+    // the launch constants are all needed within the next few hundred instructions: naming them here lets the compiler
+    // fetch them as a few wide scalar loads instead of one load and one wait per use
+    asm volatile("" : : "s"(sp.xOk), "s"(sp.xRxLog), "s"(sp.xCxLog), "s"(sp.xRowsPer), "s"(sp.xColsPer), "s"(sp.xPerRank),
+                 "s"(sp.xCommLoops), "s"(sp.xLastPerRank), "s"(sp.coreLoops), "s"(sp.loopsM), "s"(sp.loopsN), "s"(sp.blockPerComm),
+                 "s"(sp.m0), "s"(sp.n0), "s"(sp.mRank), "s"(sp.off));
+    asm volatile("" : : "s"(sp.dColsPer.d), "s"(sp.dColsPer.m), "s"(sp.dLoopsM.d), "s"(sp.dLoopsM.m), "s"(sp.dBand.d), "s"(sp.dBand.m),
+                 "s"(sp.dPerRank.d), "s"(sp.dPerRank.m), "s"(sp.dStages.d), "s"(sp.dStages.m), "s"(sp.dBpc.d), "s"(sp.dBpc.m),
+                 "s"(args.keptRank), "s"(args.flags), "s"(args.K), "s"(args.N));
     const bool linear = (args.flags & GF_LINEAR_ORDER) != 0;
     // A launch with few tiles can cut every tile's k range into kSlices pieces, one workgroup each (128-row tiles
     // only): position `pos` of the launch order runs as kSlices workgroups that stay in the position's XCD column.
