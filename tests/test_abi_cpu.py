@@ -181,6 +181,36 @@ def test_launch_tile_equals_launch_task_then_task_tile(so):
         assert so.catcoc_launch_tile(comm, C.byref(t), C.byref(d), n, None, None, None, None, None) == 0
 
 
+def test_launch_tile_random_shapes(so):
+    # the same comparison over random grids, rank counts, swizzles and round layouts (sampled workgroups)
+    from mm_rs_with_catlass_amd import ops
+    rng = np.random.default_rng(11)
+    task, tr, row, col, wsr = (u32() for _ in range(5))
+    tr2, row2, col2, wsr2 = (u32() for _ in range(4))
+    done = 0
+    for _ in range(60):
+        P = int(rng.choice([1, 2, 4, 8]))
+        comm = int(rng.choice([L.QUANT_MATMUL_REDUCE_SCATTER, L.MATMUL_REDUCE_SCATTER, L.MATMUL_ALLREDUCE]))
+        m0 = int(rng.choice([128, 256]))
+        rows_per_rank = m0 * int(rng.integers(1, 9))
+        M = rows_per_rank * (P if comm != L.MATMUL_ALLREDUCE else 1)
+        N = 256 * int(rng.integers(1, 12))
+        kw = dict(block_num=int(rng.choice([0, 4, 8, 20])) * P, stages=int(rng.integers(0, 4)),
+                  swizzle=(int(rng.integers(1, 9)), int(rng.integers(0, 2))))
+        t = ops.default_tiling(M, 512, N, P, m0=m0, n0=256, k0=256, commInterval=int(rng.integers(1, 4)))
+        d = L.make_desc(int(rng.integers(0, P)), P, **kw)
+        n = so.catcoc_get_task_count(comm, C.byref(t), C.byref(d))
+        if n == 0:
+            continue        # a layout the library rejects (it says why); nothing to compare
+        for wg in sorted(set(int(x) for x in rng.integers(0, n, 40)) | {0, n - 1}):
+            assert so.catcoc_launch_tile(comm, C.byref(t), C.byref(d), wg, C.byref(task), C.byref(tr), C.byref(row), C.byref(col), C.byref(wsr)) == 1
+            assert task.value == so.catcoc_launch_task(comm, C.byref(t), C.byref(d), wg)
+            assert so.catcoc_task_tile(comm, C.byref(t), C.byref(d), task.value, C.byref(tr2), C.byref(row2), C.byref(col2), C.byref(wsr2)) == 1
+            assert (tr.value, row.value, col.value, wsr.value) == (tr2.value, row2.value, col2.value, wsr2.value), (comm, M, N, P, m0, kw, wg)
+        done += 1
+    assert done >= 30
+
+
 def test_reciprocal_division_is_exact():
     # the formula of the schedulers' FastDiv (m = floor(2^32 / d), estimate mulhi(n, m), two corrections)
     rng = np.random.default_rng(3)
