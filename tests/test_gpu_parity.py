@@ -2,6 +2,8 @@
 seeded inputs.  Bars: int32 accumulators bit-exact; W8A8 outputs within 1 ulp of the 16-bit output
 type (the build reduces in the oracle's order, so they are normally equal); float GEMMs within
 rel-err 1e-2 of the fp32 k-sequential oracle and inside the reference's own rtol gate."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -688,3 +690,26 @@ def test_cpp_host_drives_the_library_through_the_c_abi(tmp_path):
     # a rejected launch is reported, not executed
     r = subprocess.run([exe, str(P), str(rank), str(M), str(N), str(K), str(tmp_path / "missing")], capture_output=True, text=True, timeout=100)
     assert r.returncode == 1 and "cannot read" in r.stderr
+
+
+def test_bench_prints_one_json_line_with_roofline():
+    # the measurement contract: one JSON line, whole-job throughput, the roofline object of the dominant kernel
+    _need_gpu()
+    import json
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "3", "--warmup", "1", "--no-cpu"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 3 and d["unit"] == "TOPS" and d["vs_baseline"] is None and d["dtype"] == "int8"
+    assert "workload" in d["config"] and d["config"]["parity_sample_ok"] is True
+    rf = d["roofline"]
+    assert rf["bound"] == "mfma" and rf["peak"] == 5000.0 and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3
+    assert 100.0 < d["value"] < 5000.0
