@@ -34,6 +34,10 @@
  *                                         pinned by hand-worked cases and
  *                                         bijection / rotation invariants.
  *   GetSplitkFactor, tiling search      : hand-enumerated cases.
+ *   reduce-scatter / all-reduce task    : cases worked by hand from KQ:159-201
+ *   maps, int32 peer reduce               and KAR:146-179 (several rounds, a
+ *                                         reversed narrow band); numpy with
+ *                                         distinct peers and a row offset.
  *   peer reduce order                   : defined by this build (local partial
  *                                         first, then peers in ascending slot
  *                                         order); the reference reduces with

@@ -396,6 +396,86 @@ def test_rs_task_schedule_config4():
     assert oracle.rs_task(*args, 200)[:3] == (0, 3, 4)  # loopIdxInRank 25 -> (25 // 7, 25 % 7)
 
 
+def test_ar_task_hand_worked_cases():
+    # include/catcoc/dgemm/kernel/matmul_allreduce.hpp:146-179 worked by hand.
+    # (a) BASELINE config 1 with the reference launch: 512x1024 in 128x256 tiles = 4x4 tiles, 20 cores x
+    # commInterval 3 = 60 tiles per round, so all 16 tasks are round 0 / stage 0 and tile t sits at workspace
+    # row t*128; swizzle <7,1> on 4 tile columns is a single (last, narrower) band of width 4: task -> (t/4, t%4).
+    for t in range(16):
+        assert oracle.ar_task(512, 1024, 128, 256, 20, 3, 2, t) == (t // 4, t % 4, t * 128)
+    assert oracle.ar_task(512, 1024, 128, 256, 20, 3, 2, 16) is None
+    # (b) several rounds and a narrow reversed last band: 512x2304 -> 4x9 tiles, 5 cores x commInterval 2 = 10
+    # tiles per round, 2 stages.  Band 0 = tile columns 0..6 (28 tasks, n fastest); band 1 = columns 7,8 with
+    # the tile rows walked backwards.
+    args = (512, 2304, 128, 256, 5, 2, 2)
+    assert oracle.ar_task(*args, 0) == (0, 0, 0)
+    assert oracle.ar_task(*args, 9) == (1, 2, 9 * 128)                   # round 0, b = 9
+    assert oracle.ar_task(*args, 17) == (2, 3, (10 + 7) * 128)           # round 1 -> stage 1, b = 7
+    assert oracle.ar_task(*args, 23) == (3, 2, 3 * 128)                  # round 2 -> stage 0 again, b = 3
+    assert oracle.ar_task(*args, 28) == (3, 7, (0 + 8) * 128)            # first task of the reversed band
+    assert oracle.ar_task(*args, 29) == (3, 8, (0 + 9) * 128)
+    assert oracle.ar_task(*args, 30) == (2, 7, (10 + 0) * 128)           # round 3 -> stage 1
+    assert oracle.ar_task(*args, 35) == (0, 8, (10 + 5) * 128)
+    assert oracle.ar_task(*args, 36) is None
+    assert len({oracle.ar_task(*args, t)[:2] for t in range(36)}) == 36
+
+
+def test_splitk_slices_hand_worked_case():
+    # block_swizzle.hpp:151-158,220-235 by hand: 9 k tiles over 4 slices -> the FIRST 9 % 4 = 1 slice owns one
+    # extra tile: slices start at k tiles 0, 3, 5, 7 and hold 3, 2, 2, 2 tiles; the last slice's extent is what
+    # is left of K (ragged K = 9*256 - 100).
+    assert [oracle.lib().oracle_splitk_first_ktile(u32(9), u32(4), u32(s)) for s in range(4)] == [0, 3, 5, 7]
+    K = 9 * 256 - 100
+    assert [oracle.splitk_actual_k(K, 256, 4, s) for s in range(4)] == [768, 512, 512, K - 7 * 256]
+    # 10 k tiles over 4: two slices with an extra tile -> starts 0, 3, 6, 8
+    assert [oracle.lib().oracle_splitk_first_ktile(u32(10), u32(4), u32(s)) for s in range(4)] == [0, 3, 6, 8]
+    # task -> (m, n, first k tile, slice) on a 2x3 tile grid, swizzle <7,1> (one band of width 3: m = i/3, n = i%3):
+    # the slice is the task's index divided by the 6 tiles of the grid
+    assert oracle.splitk_block_coord(7, 1, 2, 3, 9, 4, 13) == (0, 1, 5, 2)
+    assert oracle.splitk_block_coord(7, 1, 2, 3, 9, 4, 23) == (1, 2, 7, 3)
+    assert oracle.splitk_block_coord(7, 1, 2, 3, 9, 4, 5) == (1, 2, 0, 0)
+    assert oracle.splitk_block_coord(7, 1, 2, 3, 9, 4, 24 + 6) == (0, 0, 3, 1)    # wraps modulo the 24 tasks
+
+
+def test_allgather_swizzle_hand_worked_ragged_last_round():
+    # include/catcoc/dgemm/block/block_swizzle_allgather.hpp:88-108 by hand: P = 2 ranks with 3 tile rows each,
+    # 2 tile columns, commInterval 2 -> rounds of 4 tile rows (2 per rank), then a last round of 2 (1 per rank).
+    # Inside a round the base swizzle <7,1> on 2 columns is one band of width 2: (cm, cn) = (i/2, i%2); the row is
+    # re-based rank-major: m = rank*3 + round*2 + cm % rowsPerRankThisRound.
+    f = lambda t: oracle.allgather_block_coord(7, 1, 2, 2, 3, 2, t)
+    assert f(0) == (0, 0) and f(3) == (1, 1)
+    assert f(4) == (3, 0) and f(5) == (3, 1) and f(7) == (4, 1)      # second half of round 0 = rank 1
+    assert f(8) == (2, 0) and f(9) == (2, 1)                          # last round: one row per rank
+    assert f(10) == (5, 0) and f(11) == (5, 1)
+    assert sorted(f(t) for t in range(12)) == [(m, n) for m in range(6) for n in range(2)]
+    # direction 0, band width 3 on the 4 rows of round 0: band 0 = rows 0..2 (m fastest), band 1 = row 3 with the
+    # columns walked backwards
+    g = lambda t: oracle.allgather_block_coord(3, 0, 2, 2, 3, 2, t)
+    assert [g(t) for t in range(8)] == [(0, 0), (1, 0), (3, 0), (0, 1), (1, 1), (3, 1), (4, 1), (4, 0)]
+
+
+def test_reduce_i32_distinct_peers_and_row_offset():
+    rng = np.random.default_rng(11)
+    M, N, ld, r0 = 5, 7, 9, 3
+    acc = rng.integers(-10 ** 6, 10 ** 6, (M, N), dtype=np.int32)
+    peers = [rng.integers(-10 ** 6, 10 ** 6, (M + r0 + 2, ld), dtype=np.int32) for _ in range(3)]
+    got = acc.copy()
+    arr = (C.c_void_p * 3)(*[p.ctypes.data for p in peers])
+    oracle.lib().oracle_reduce_i32(u32(M), u32(N), _p(got), C.c_int64(N), u32(3), arr, C.c_int64(ld), C.c_int64(r0))
+    want = acc + sum(p[r0:r0 + M, :N] for p in peers)
+    assert np.array_equal(got, want)
+    # through the whole-operator entry: int32 peers with a row offset against numpy
+    x1 = rng.integers(-127, 128, (8, 16), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (16, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, 8).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    pk = [rng.integers(-10 ** 5, 10 ** 5, (2 + r0, N), dtype=np.int32) for _ in range(3)]
+    _, out = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, 4, 2, pk, oracle.FP16, peer_row0=r0, reduce_int32=True)
+    tot = (x1[4:6].astype(np.int64) @ x2.astype(np.int64) + sum(p[r0:r0 + 2].astype(np.int64) for p in pk)).astype(np.int32)
+    want = ((tot.astype(np.float32) * s2[None, :]) * s1[4:6, None]).astype(np.float16)
+    assert np.array_equal(out, want.view(np.uint16))
+
+
 def test_tiling_search_space():
     base = oracle.TilingParams(m=8192, k=1792, n=4096, m0=128, k0=256, n0=256, commTileM=64, commInterval=20,
                                commNpuSplit=1, commDataSplit=2, commBlockM=64, rankSize=8)
