@@ -6,7 +6,7 @@ BASELINE config 4, A[8192,1792] int8, B[1792,4096] int8, per-token / per-channel
 7 staged fp32 peer partials of the kept block, kept output [1024,4096] bf16.  Inputs are resident
 in HBM before the timed region.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode kept|outbound] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode kept|outbound] [--no-cpu] [--sets S] [--sustained L]
     python bench.py --mode copy     # plain 256 MiB device copy: the known-size kernel the HBM counters are scaled by
     python bench.py --mode decode   # BASELINE config 5: skinny-M sweep, K = N = 8192, GB/s per M (HBM-bound)
     python bench.py --mode float    # BASELINE configs 3 (fp16 reduce-scatter), 2 (bf16 all-gather) and 1 (fp16 all-reduce)
@@ -105,6 +105,9 @@ def decode_sweep(args, torch, L, ops, dev):
         "roofline": {"bound": "hbm", "achieved": worst["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(worst["GBps"] / PEAK_HBM_GBS, 4), "traffic": None},
         "sweep": sweep}))
+    if not all(r["parity_ok"] for r in sweep):
+        print("bench.py: a decode-sweep output does NOT match the oracle", file=sys.stderr)
+        sys.exit(3)
 
 
 PEAK_F16_TFLOPS = 2500.0   # MI355X dense fp16 / bf16 MFMA, published
@@ -181,6 +184,9 @@ def float_configs(args, torch, L, ops, dev):
         "roofline": {"bound": "mfma", "achieved": c3["TFLOPS"], "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(c3["TFLOPS"] / PEAK_F16_TFLOPS, 4), "traffic": None},
         "configs": res}))
+    if not rel <= 1e-2:
+        print("bench.py: the config-3 row sample is off by %g from the oracle" % rel, file=sys.stderr)
+        sys.exit(3)
 
 
 def main():
@@ -195,6 +201,9 @@ def main():
     ap.add_argument("--cpu-repeats", type=int, default=5)
     ap.add_argument("--rank", type=int, default=0)
     ap.add_argument("--m0", type=int, default=0)
+    ap.add_argument("--sets", type=int, default=4, help="independent input sets the launches rotate over (1 = same buffers every launch)")
+    ap.add_argument("--sustained", type=int, default=300, help="launches of the untimed sustained block (0 = skip)")
+    ap.add_argument("--no-other-mode", action="store_true", help="skip the secondary run of the other store mode")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (peers are staged in the same GPU's HBM); --gpus %d is not "
@@ -233,68 +242,109 @@ def main():
         return
     M, K, N, P, rank = 8192, 1792, 4096, 8, args.rank
     rows = M // P
-    g = torch.Generator(device=dev).manual_seed(20250101)
-    x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
-    x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
-    s1 = torch.empty(M, device=dev).uniform_(0.005, 0.02, generator=g)
-    s2 = torch.empty(N, device=dev).uniform_(0.001, 0.01, generator=g)
-    peers = [torch.randn((rows, N), device=dev, generator=g) for _ in range(P - 1)]
-    out = torch.empty((rows, N), dtype=torch.bfloat16, device=dev)
     tiling = ops.default_tiling(M, K, N, P, m0=args.m0, n0=0, k0=0)
     desc0 = L.make_desc(rank, P, [16] * (P - 1))
-    ntasks = L.load().catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(tiling), C.byref(desc0))
-    kw = {}
-    if args.mode == "outbound":
-        need = L.load().catcoc_get_workspace_size(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, C.byref(tiling), C.byref(desc0))
-        kw["outbound"] = torch.empty(need // 4, dtype=torch.float32, device=dev)
-    else:
-        kw["checksum"] = torch.zeros(ntasks, dtype=torch.int64, device=dev)
+    so = L.load()
+    ntasks = so.catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(tiling), C.byref(desc0))
+    ob_bytes = so.catcoc_get_workspace_size(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, C.byref(tiling), C.byref(desc0))
 
-    # arguments are validated and bound once; a step is one call of the C-ABI launcher
-    step, _ = ops.prepare_quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, rank, P, tiling=tiling, out=out, **kw)
-    step()
-    L.check()
+    # Input sets.  A launch reads 148 MB; replaying one set back to back lets the 256 MB Infinity Cache serve part of it,
+    # which a real reduce-scatter (fresh activations, freshly written peer partials) never sees.  The timed steps therefore
+    # rotate over `--sets` independent sets (default 4 = 592 MB), so every launch reads its operands from HBM; the
+    # same-buffer figure is reported next to it as "hot".
+    g = torch.Generator(device=dev).manual_seed(20250101)
+    sets = []
+    for _ in range(max(1, args.sets)):
+        x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
+        x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
+        s1 = torch.empty(M, device=dev).uniform_(0.005, 0.02, generator=g)
+        s2 = torch.empty(N, device=dev).uniform_(0.001, 0.01, generator=g)
+        peers = [torch.randn((rows, N), device=dev, generator=g) for _ in range(P - 1)]
+        out = torch.empty((rows, N), dtype=torch.bfloat16, device=dev)
+        sets.append(dict(x1=x1, x2=x2, s1=s1, s2=s2, peers=peers, out=out))
+    outbound = torch.empty(ob_bytes // 4, dtype=torch.float32, device=dev)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    # HIP events on the launch stream (torch's current stream) bracket the K launches inside the timed region;
-    # the launches queue back to back, so elapsed / K is the kernel's average duration
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(args.steps):
-        step()
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    avg_kernel_s = e0.elapsed_time(e1) / args.steps / 1e3
-    ms_per_step = wall / args.steps * 1e3
-    # untimed extra pass with one event pair per launch, for the spread (each pair adds the events' own cost, so its
-    # minimum can sit above the back-to-back average)
+    def prepare(mode):
+        """One bound launch per input set: arguments are validated once; a step is one call of the C-ABI launcher."""
+        steps = []
+        for st in sets:
+            kw = {"outbound": outbound} if mode == "outbound" else {"checksum": torch.zeros(ntasks, dtype=torch.int64, device=dev)}
+            fn, _ = ops.prepare_quant_matmul_reduce_scatter(st["x1"], st["x2"], st["s1"], st["s2"], None, st["peers"], rank, P,
+                                                            tiling=tiling, out=st["out"], **kw)
+            steps.append(fn)
+        steps[0]()
+        L.check()
+        return steps
+
+    def run(steps, n, first=0):
+        """n launches queued back to back on torch's current stream, bracketed by HIP events on that stream.
+        -> (wall seconds per launch, kernel seconds per launch)"""
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(n):
+            steps[(first + i) % len(steps)]()
+        e1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n, e0.elapsed_time(e1) / n / 1e3
+
+    main_steps = prepare(args.mode)
+    for i in range(args.warmup):
+        main_steps[i % len(main_steps)]()
+    # ---- the timed region: exactly K steps between two synchronisations -------------------------------------
+    wall_s, avg_kernel_s = run(main_steps, args.steps, first=args.warmup)
+    ms_per_step = wall_s * 1e3
+    last_set = sets[(args.warmup + args.steps - 1) % len(sets)]
+    kept_bits = last_set["out"].view(torch.int16).clone()
+
+    # ---- untimed extras -----------------------------------------------------------------------------------------
+    # the same buffers over and over ("hot": part of the operands comes from the Infinity Cache)
+    _, hot_kernel_s = run(main_steps[:1], args.steps)
+    # a long block: sustained launches are power-limited and slower than the first few dozen; ten event-bracketed
+    # groups of `--sustained`/10 launches show the curve
+    grp = max(1, args.sustained // 10)
+    series = [run(main_steps, grp, first=j * grp)[1] for j in range(10)] if args.sustained > 0 else []
+    # one event pair per launch, for the spread
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(min(args.steps, 20))]
-    for a, b in evs:
+    for i, (a, b) in enumerate(evs):
         a.record()
-        step()
+        main_steps[i % len(main_steps)]()
         b.record()
     torch.cuda.synchronize()
     kern_ms = [a.elapsed_time(b) for a, b in evs]
+
+    # the other store mode, as a secondary object: the reference stores the 7/8 non-kept tiles for its peers to pull
+    other_mode = "kept" if args.mode == "outbound" else "outbound"
+    other = None
+    if not args.no_other_mode:
+        other_steps = prepare(other_mode)
+        for i in range(args.warmup):
+            other_steps[i % len(other_steps)]()
+        o_wall, o_kern = run(other_steps, args.steps, first=args.warmup)
+        same = bool(torch.equal(kept_bits, last_set["out"].view(torch.int16)))   # same set, same kept block, bit for bit
+        o_bytes = M * K + K * N + 4 * (M + N) + (P - 1) * rows * N * 4 + rows * N * 2 + ((P - 1) * rows * N * 4 if other_mode == "outbound" else 0)
+        other = {"mode": other_mode, "ms_per_step": round(o_wall * 1e3, 5), "kernel_us_avg": round(o_kern * 1e6, 2),
+                 "TOPS": round(2.0 * M * N * K / o_kern / 1e12, 2), "mfma_frac": round(2.0 * M * N * K / o_kern / 1e12 / PEAK_INT8_TOPS, 4),
+                 "algorithmic_bytes": int(o_bytes), "hbm_frac": round(o_bytes / o_kern / 1e9 / PEAK_HBM_GBS, 4),
+                 "kept_block_equals_main_mode": same}
 
     # bounded parity check of the timed configuration: a row sample of the kept block against the oracle
     import numpy as np
     import oracle
     sel = np.arange(0, rows, 97)
+    st = last_set
     _, want = oracle.quant_matmul_reduce_scatter(
-        x1[rank * rows + sel].cpu().numpy(), x2.cpu().numpy(), s1[rank * rows + sel].cpu().numpy(), s2.cpu().numpy(),
-        None, 0, len(sel), [p[sel].cpu().numpy() for p in peers], oracle.BF16, want_acc=False)
-    got = out[sel].view(torch.int16).cpu().numpy().view(np.uint16)
-    parity_ok = bool(np.array_equal(got, want))
+        st["x1"][rank * rows + sel].cpu().numpy(), st["x2"].cpu().numpy(), st["s1"][rank * rows + sel].cpu().numpy(),
+        st["s2"].cpu().numpy(), None, 0, len(sel), [p[sel].cpu().numpy() for p in st["peers"]], oracle.BF16, want_acc=False)
+    got = kept_bits[sel].cpu().numpy().view(np.uint16)
+    parity_ok = bool(np.array_equal(got, want)) and (other is None or other["kept_block_equals_main_mode"])
 
     ops_per_step = 2.0 * M * N * K
     alg_bytes = M * K + K * N + 4 * (M + N) + (P - 1) * rows * N * 4 + rows * N * 2
     if args.mode == "outbound":
         alg_bytes += (P - 1) * rows * N * 4
-    value = ops_per_step / (wall / args.steps) / 1e12
+    value = ops_per_step / wall_s / 1e12
     achieved = ops_per_step / avg_kernel_s / 1e12
     info = ops.device_info()
     traffic = None
@@ -304,6 +354,7 @@ def main():
             traffic = json.load(open(tpath)).get("quant_rs_config4_" + args.mode)
         except Exception:
             traffic = None
+    sustained_s = sum(series[5:]) / len(series[5:]) if series else None
     line = {
         "metric": "W8A8 matmul-RS shard int8 TOPS + % MFMA/HBM roofline, 1 MI355X",
         "value": round(value, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -312,17 +363,29 @@ def main():
         "config": {"workload": "W8A8 quant matmul-reduce-scatter shard (BASELINE config 4): M=8192 K=1792 N=4096 "
                                "P=8 rank=%d, int8 x int8 -> int32, dequant, +7 staged fp32 peers, bf16 [1024,4096]" % rank,
                    "mode": args.mode, "tile": "%dx256x64" % (tiling.m0 or 128), "tasks": int(ntasks),
-                   "parity_sample_ok": parity_ok},
+                   "input_sets_rotated": len(sets), "parity_sample_ok": parity_ok},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": traffic,
-                     "kernel_us_avg": round(avg_kernel_s * 1e6, 2), "single_launch_us_min": round(min(kern_ms) * 1e3, 2),
+                     "kernel_us_avg": round(avg_kernel_s * 1e6, 2),
+                     "kernel_us_avg_same_buffers": round(hot_kernel_s * 1e6, 2),
+                     "kernel_us_sustained": round(sustained_s * 1e6, 2) if sustained_s else None,
+                     "frac_sustained": round(ops_per_step / sustained_s / 1e12 / PEAK_INT8_TOPS, 4) if sustained_s else None,
+                     "sustained_series_us": [round(x * 1e6, 2) for x in series],
+                     "sustained_note": "%d more launches in ten event-bracketed groups after the timed steps; "
+                                       "kernel_us_sustained = mean of the last five groups" % (grp * 10) if series else None,
+                     "single_launch_us_min": round(min(kern_ms) * 1e3, 2),
                      "algorithmic_bytes": int(alg_bytes),
                      "hbm_frac_at_algorithmic_bytes": round(alg_bytes / avg_kernel_s / 1e9 / PEAK_HBM_GBS, 4)},
         "device": info,
     }
+    if other is not None:
+        line[other_mode] = other
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(M, N, K, P, rank, args.cpu_repeats)
     print(json.dumps(line))
+    if not parity_ok:
+        print("bench.py: the parity sample of the timed configuration does NOT match the oracle", file=sys.stderr)
+        sys.exit(3)
 
 
 if __name__ == "__main__":

@@ -82,6 +82,7 @@ typedef void (*CatcocKernelFuncPtr)(void *stream, uint64_t fftsAddr, uint8_t *a,
 /* ----------------------------------------------------------------------- */
 
 #define CATCOC_MAX_RANKS 16
+#define CATCOC_WORKSPACE_COUNTER_BYTES 65536u /* counter block at the start of CatcocSymmetricDesc.workspace */
 #define CATCOC_DESC_MAGIC 0x43544343u /* "CCTC" */
 
 /* What happens to tiles whose rows belong to another rank (the reference stores
@@ -130,9 +131,12 @@ typedef struct CatcocSymmetricDesc {
     void *accDump;            /* optional full [m,n] int32 (W8A8) or fp32 (float) local partial, for bit-exact checks */
     /* Scratch in HBM for launches whose k range is cut into slices: the skinny-M split-K path
      * (catcoc_get_splitk_workspace_size() bytes) and few-tile launches of the large-tile kernel
-     * (catcoc_get_kslice_workspace_size() bytes, optional there).  256-byte aligned, ZEROED by the caller once
-     * before its first use (the library leaves it re-armed after every launch).  Launches that share a workspace
-     * must not overlap (same stream, or ordered by events). */
+     * (catcoc_get_kslice_workspace_size() bytes, optional there).  256-byte aligned.  Layout: the first
+     * CATCOC_WORKSPACE_COUNTER_BYTES hold one arrival counter per tile, at the same place for every shape and slice
+     * count; the partial tiles follow.  The caller ZEROES the counter block (or simply the whole buffer) once before
+     * the first use; every launch leaves the counters at zero again, so launches of any shapes may share one
+     * workspace that is large enough for each of them.  Launches that share a workspace must not overlap (same
+     * stream, or ordered by events). */
     void *workspace;
     uint64_t workspaceBytes;
 } CatcocSymmetricDesc;

@@ -57,6 +57,11 @@ enum { E_NULL = 1, E_DESC = 2, E_SHAPE = 3, E_RANK = 4, E_TILING = 5, E_DTYPE = 
 
 constexpr uint32_t kDefaultBlockNum = 256;  // one scheduling slot per CU of an MI355X
 constexpr uint32_t kDefaultStages = 2;      // WORKSPACE_STAGES, examples/dynamic_tiling/include/info.h:18
+// Every workspace starts with one block of per-tile arrival counters at a fixed place and of a fixed size, whatever the
+// shape or slice count of the launch: launches of different shapes can then share one workspace that was zeroed once
+// (each launch leaves its counters at zero again; the partial tiles behind the block are written before they are read).
+constexpr uint64_t kCounterBlockBytes = CATCOC_WORKSPACE_COUNTER_BYTES;
+constexpr uint32_t kMaxCountedTiles = (uint32_t)(kCounterBlockBytes / 4u);
 
 struct Plan {
     GemmArgs args;
@@ -213,15 +218,16 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
         }
         if (f > 1) {
             plan.kSlices = f;
-            plan.kSliceBytes = (uint64_t)T * f * (128u * 256u * 4u) + (((uint64_t)T * 4u + 255u) & ~255ull);
+            if (T > kMaxCountedTiles) return fail(E_TILING, "k slices: %u tiles exceed the %u the workspace counts", T, kMaxCountedTiles);
+            plan.kSliceBytes = kCounterBlockBytes + (uint64_t)T * f * (128u * 256u * 4u);
             if (d->workspace != nullptr) {
                 if ((uintptr_t)d->workspace % 256 != 0) return fail(E_WORKSPACE, "workspace must be 256-byte aligned");
                 if (d->workspaceBytes < plan.kSliceBytes)
                     return fail(E_WORKSPACE, "workspace too small for %u k slices: %llu < %llu bytes", f,
                                 (unsigned long long)d->workspaceBytes, (unsigned long long)plan.kSliceBytes);
                 a.splitK = f;
-                a.skPart = (int32_t *)d->workspace;
-                a.skCount = (uint32_t *)((unsigned char *)d->workspace + (uint64_t)T * f * (128u * 256u * 4u));
+                a.skCount = (uint32_t *)d->workspace;
+                a.skPart = (int32_t *)((unsigned char *)d->workspace + kCounterBlockBytes);
             } else if (d->splitK != 0) {
                 return fail(E_WORKSPACE, "splitK %u needs a workspace of %llu bytes", f, (unsigned long long)plan.kSliceBytes);
             }
@@ -322,7 +328,9 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
     sp.f = f;
     a.splitK = f;
     sp.rowBlocks = t->m <= 32 ? 1 : t->m <= 64 ? 2 : 4;
-    sp.workspaceBytes = f > 1 ? (uint64_t)f * sp.tiles * 128u * 128u * 4u + (uint64_t)((sp.tiles * 4u + 255u) / 256u) * 256u : 0;
+    if (f > 1 && sp.tiles > kMaxCountedTiles)
+        return fail(E_TILING, "split-K: %u tiles exceed the %u the workspace counts", sp.tiles, kMaxCountedTiles);
+    sp.workspaceBytes = f > 1 ? kCounterBlockBytes + (uint64_t)f * sp.tiles * 128u * 128u * 4u : 0;
     return 0;
 }
 
@@ -346,8 +354,8 @@ void launch_quant_splitk(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_
             return;
         }
         if ((uintptr_t)d->workspace % 256 != 0) { fail(E_WORKSPACE, "workspace must be 256-byte aligned"); return; }
-        a.skPart = (int32_t *)d->workspace;
-        a.skCount = (uint32_t *)((unsigned char *)d->workspace + (uint64_t)sp.f * sp.tiles * 128u * 128u * 4u);
+        a.skCount = (uint32_t *)d->workspace;
+        a.skPart = (int32_t *)((unsigned char *)d->workspace + kCounterBlockBytes);
     }
     a.a[0] = x1;
     a.b = x2;

@@ -3,18 +3,6 @@
 // MFMAs, and the row-major B tile is transposed on the way out of LDS with the
 // transpose-read instruction, so the main loop issues almost nothing but LDS reads
 // and MFMAs.
-//
-// Reduce-scatter launches have few kept tiles, and each of them has to add the peers'
-// partials for its rows (0.9 MB per tile at 128x256 with 7 peers), which takes longer
-// than the tile's main loop and keeps its slot on the CU busy while the rest of the
-// launch runs out of work to pack around it.  With a workspace the kept tiles only
-// publish their dequantised fp32 tile and leave; the workgroups of the second half of
-// the launch each add the peers for one slice of the kept block after their own tile,
-// in the same order per element (local, then peers in slot order), so the result is
-// bit-identical and the reduce work is spread evenly over every slot.  A slice is
-// finished on the XCD that published it: the values then travel through that XCD's L2
-// with ordinary stores (device-scope write-through stores of this volume measured
-// 50 GB/s).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -717,9 +705,9 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         Sum si = 0;
         bool summed = false;
         if constexpr (DT == DT_I8) {
-            // |accumulator| <= 127 * 127 * k, so without a bias four of them add in 32 bits for k <= 32768: a third of
-            // the 64-bit additions
-            if (args.bias == nullptr && args.K <= 32768u) {
+            // |accumulator| <= 128 * 128 * k (int8 admits -128), so without a bias four of them add in 32 bits for
+            // k < 32768 (4 * 2^14 * 32767 < 2^31): a third of the 64-bit additions
+            if (args.bias == nullptr && args.K < 32768u) {
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll

@@ -15,6 +15,7 @@ INT8 = 2
 BF16 = 27
 
 MAX_RANKS = 16
+WORKSPACE_COUNTER_BYTES = 65536
 DESC_MAGIC = 0x43544343
 OUTBOUND_CHECKSUM = 0
 OUTBOUND_STORE = 1
@@ -106,7 +107,8 @@ def load():
     u32, vp = C.c_uint32, C.c_void_p
     pu = C.POINTER(u32)
     for name in EXPORTS:
-        if name.startswith("catcoc_launch_") and name != "catcoc_launch_quant_matmul_reduce_scatter":
+        if name.startswith("catcoc_launch_") and not name.startswith("catcoc_launch_quant_") and name not in (
+                "catcoc_launch_task", "catcoc_launch_tile"):
             f = getattr(L, name)
             f.argtypes = _LAUNCHER_ARGS
             f.restype = None

@@ -47,6 +47,47 @@ def _check_dev(*ts):
             raise _l.CatcocError("operands must be contiguous")
 
 
+def _fail(msg, *a):
+    raise _l.CatcocError(msg % a if a else msg)
+
+
+def _want(t, name, dtype=None, ndim=None, numel=None, shape=None):
+    """One operand against what the kernels will read or write: the C ABI sees raw pointers only, so sizes and element
+    types can be checked here and nowhere else (a short or mistyped buffer is an out-of-bounds access on the GPU)."""
+    if t is None:
+        return
+    if dtype is not None and t.dtype not in (dtype if isinstance(dtype, tuple) else (dtype,)):
+        _fail("%s must be %s (got %s)", name, dtype, t.dtype)
+    if ndim is not None and t.dim() != ndim:
+        _fail("%s must have %d dimensions (got shape %s)", name, ndim, tuple(t.shape))
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        _fail("%s must have shape %s (got %s)", name, tuple(shape), tuple(t.shape))
+    if numel is not None and t.numel() < numel:
+        _fail("%s holds %d elements, the launch needs %d", name, t.numel(), numel)
+
+
+def _check_peers(peers, count, dtype, rows_needed, n, what="peers"):
+    if len(peers) != count:
+        _fail("%s: %d buffers given, rank_size - 1 = %d needed", what, len(peers), count)
+    for i, p in enumerate(peers):
+        _want(p, "%s[%d]" % (what, i), dtype, 2)
+        if p.shape[1] != peers[0].shape[1]:
+            _fail("%s[%d] has %d columns, %s[0] has %d: one leading dimension serves all", what, i, p.shape[1], what, peers[0].shape[1])
+        if p.shape[1] < n or p.shape[0] < rows_needed:
+            _fail("%s[%d] has shape %s, the launch reads rows [0,%d) x %d columns", what, i, tuple(p.shape), rows_needed, n)
+
+
+def _check_rank(rank, rank_size):
+    if rank_size < 1 or rank_size > _l.MAX_RANKS or not 0 <= rank < rank_size:
+        _fail("rank %d / rank_size %d out of range (1..%d ranks)", rank, rank_size, _l.MAX_RANKS)
+
+
+def _task_count(comm_type, t, d):
+    n = int(_l.load().catcoc_get_task_count(comm_type, C.byref(t), C.byref(d)))
+    _l.check()
+    return n
+
+
 def _attach_workspace(d, workspace, split_k):
     """Optional scratch for k-sliced launches (kslice_plan() says how large) and the caller's own slice count."""
     d.splitK = split_k
@@ -71,16 +112,38 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
                                         out=None, workspace=None, split_k=0):
     """Validate and bind the arguments once; returns (launch, out) where launch() enqueues one call of
     catcoc_launch_quant_matmul_reduce_scatter on torch's current stream (for launch-rate-sensitive loops)."""
-    _check_dev(x1, x2, scale_x1, scale_x2, bias, outbound, checksum, acc_dump, c_accum, *peers)
+    _check_rank(rank, rank_size)
+    _want(x1, "x1", torch.int8, 2)
+    _want(x2, "x2", torch.int8, 2)
     m, k = x1.shape
     n = x2.shape[0] if trans_b else x2.shape[1]
+    if (x2.shape[1] if trans_b else x2.shape[0]) != k:
+        _fail("x2 has shape %s: its k extent does not match x1's k = %d", tuple(x2.shape), k)
+    if m % rank_size != 0:
+        _fail("reduce-scatter needs m %% rank_size == 0 (m=%d, rank_size=%d)", m, rank_size)
+    if peer_row_offset < 0:
+        _fail("peer_row_offset must be >= 0")
+    rows = m // rank_size
+    _want(scale_x1, "scale_x1", torch.float32, 1, m)
+    _want(scale_x2, "scale_x2", torch.float32, 1, n)
+    _want(bias, "bias", torch.int32, 1, n)
+    _check_peers(list(peers), rank_size - 1, torch.int32 if reduce_int32 else torch.float32, peer_row_offset + rows, n)
+    _want(c_accum, "c_accum", torch.int32, None, rows * n)
+    _want(acc_dump, "acc_dump", torch.int32, None, m * n)
+    _want(outbound, "outbound", (torch.float32, torch.int32))
     t = tiling if tiling is not None else default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
+    if (t.m, t.k, t.n) != (m, k, n):
+        _fail("tiling says m,k,n = %d,%d,%d; the operands say %d,%d,%d", t.m, t.k, t.n, m, k, n)
     flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_REDUCE_INT32 if reduce_int32 else 0) | \
         (_l.FLAG_LINEAR_ORDER if linear_order else 0)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
     _attach_workspace(d, workspace, split_k)
+    if checksum is not None:
+        _want(checksum, "checksum", torch.int64, None, _task_count(_l.QUANT_MATMUL_REDUCE_SCATTER, t, d))
     if out is None:
-        out = torch.empty((m // max(rank_size, 1), n), dtype=out_dtype, device=x1.device)
+        out = torch.empty((rows, n), dtype=out_dtype, device=x1.device)
+    _want(out, "out", (torch.float16, torch.bfloat16), 2, None, (rows, n))
+    _check_dev(x1, x2, scale_x1, scale_x2, bias, outbound, checksum, acc_dump, c_accum, out, *peers)
     L = _l.load()
     keep = (x1, x2, scale_x1, scale_x2, bias, tuple(peers), outbound, checksum, acc_dump, c_accum, out, d, t, workspace)
     fn = L.catcoc_launch_quant_matmul_reduce_scatter
@@ -130,9 +193,27 @@ def prepare_quant_matmul_splitk(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
                                 acc_dump=None, c_accum=None, peer_row_offset=0, block_num=0, swizzle=None, out=None):
     """Skinny-M (decode) form of the W8A8 operator: x1 [m,k] with any m, the rank keeps rows
     [kept_row_begin, +kept_rows); peers are rank_size-1 fp32 partials [kept_rows, n].  Returns (launch, out)."""
-    _check_dev(x1, x2, scale_x1, scale_x2, bias, checksum, acc_dump, c_accum, workspace, *peers)
+    _check_rank(0, rank_size)
+    _want(x1, "x1", torch.int8, 2)
+    _want(x2, "x2", torch.int8, 2)
     m, k = x1.shape
     n = x2.shape[1]
+    if x2.shape[0] != k:
+        _fail("x2 has shape %s: its k extent does not match x1's k = %d", tuple(x2.shape), k)
+    kr = kept_rows if kept_rows is not None else m
+    if kept_row_begin < 0 or kr < 1 or kept_row_begin + kr > m:
+        _fail("kept rows [%d,+%d) outside [0,%d)", kept_row_begin, kr, m)
+    if peer_row_offset < 0:
+        _fail("peer_row_offset must be >= 0")
+    _want(scale_x1, "scale_x1", torch.float32, 1, m)
+    _want(scale_x2, "scale_x2", torch.float32, 1, n)
+    _want(bias, "bias", torch.int32, 1, n)
+    _check_peers(list(peers), rank_size - 1, torch.float32, peer_row_offset + kr, n)
+    _want(c_accum, "c_accum", torch.int32, None, kr * n)
+    _want(acc_dump, "acc_dump", torch.int32, None, m * n)
+    _want(checksum, "checksum", torch.int64, None, -(-m // 128) * -(-n // 128))
+    _want(out, "out", (torch.float16, torch.bfloat16), 2, None, (kr, n))
+    _check_dev(x1, x2, scale_x1, scale_x2, bias, checksum, acc_dump, c_accum, workspace, out, *peers)
     t = default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
     d = _desc(0, rank_size, list(peers), peer_row_offset, 0, block_num, 0, swizzle, None, checksum, acc_dump)
     d.keptRowBegin = kept_row_begin
@@ -164,17 +245,42 @@ def quant_matmul_splitk(*args, **kw):
 
 def _float_op(comm_type, a, b, c_shape, peers, rank, rank_size, tiling, trans_a, trans_b, peer_row_offset, outbound,
               checksum, acc_dump, block_num, stages, swizzle, linear_order, out, m_for_tiling, workspace=None, split_k=0):
-    _check_dev(a, b, outbound, checksum, acc_dump, *peers)
     if a.dtype not in _TORCH_TO_DT or b.dtype != a.dtype:
         raise _l.CatcocError("a and b must both be float16 or both bfloat16")
+    _check_rank(rank, rank_size)
+    _want(a, "a", None, 2)
+    _want(b, "b", None, 2)
     k = a.shape[0] if trans_a else a.shape[1]
     n = b.shape[0] if trans_b else b.shape[1]
+    if (b.shape[1] if trans_b else b.shape[0]) != k:
+        _fail("b has shape %s: its k extent does not match a's k = %d", tuple(b.shape), k)
+    if peer_row_offset < 0:
+        _fail("peer_row_offset must be >= 0")
+    out_shape = c_shape(n)
+    if comm_type == _l.ALLGATHER_MATMUL:
+        _check_peers(list(peers), rank_size - 1, a.dtype, a.shape[0], k, "peer_shards")
+        for i, p in enumerate(peers):
+            if tuple(p.shape) != tuple(a.shape):
+                _fail("peer_shards[%d] has shape %s, this rank's shard %s", i, tuple(p.shape), tuple(a.shape))
+    else:
+        if comm_type == _l.MATMUL_REDUCE_SCATTER and m_for_tiling % rank_size != 0:
+            _fail("reduce-scatter needs m %% rank_size == 0 (m=%d, rank_size=%d)", m_for_tiling, rank_size)
+        _check_peers(list(peers), rank_size - 1, torch.float32, peer_row_offset + out_shape[0], n)
+    rows_all = m_for_tiling * (rank_size if comm_type == _l.ALLGATHER_MATMUL else 1)
+    _want(acc_dump, "acc_dump", torch.float32, None, rows_all * n)
+    _want(outbound, "outbound", torch.float32)
     t = tiling if tiling is not None else default_tiling(m_for_tiling, k, n, rank_size, m0=0, n0=0, k0=0)
+    if (t.m, t.k, t.n) != (m_for_tiling, k, n):
+        _fail("tiling says m,k,n = %d,%d,%d; the operands say %d,%d,%d", t.m, t.k, t.n, m_for_tiling, k, n)
     flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_LINEAR_ORDER if linear_order else 0)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
     _attach_workspace(d, workspace, split_k)
+    if checksum is not None:
+        _want(checksum, "checksum", torch.float64, None, _task_count(comm_type, t, d))
     if out is None:
-        out = torch.empty(c_shape(n), dtype=a.dtype, device=a.device)
+        out = torch.empty(out_shape, dtype=a.dtype, device=a.device)
+    _want(out, "out", a.dtype, 2, None, out_shape)
+    _check_dev(a, b, outbound, checksum, acc_dump, out, *peers)
     L = _l.load()
     fn = L.catcoc_get_kernel(comm_type, _TORCH_TO_DT[a.dtype])
     if not fn:

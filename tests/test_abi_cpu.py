@@ -252,21 +252,21 @@ def test_workspace_size_queries(so):
     from mm_rs_with_catlass_amd import ops
     import torch
     # k slices of few-tile launches: fill the CUs once, at least eight k steps per slice, two slices at most for floats
-    assert ops.kslice_plan(L.ALLGATHER_MATMUL, torch.bfloat16, 512, 4096, 1024, 0, 8) == (128 * 2 * 131072 + 512, 2)
-    assert ops.kslice_plan(L.MATMUL_ALLREDUCE, torch.float16, 512, 1024, 1024, 0, 2) == (16 * 2 * 131072 + 256, 2)
+    assert ops.kslice_plan(L.ALLGATHER_MATMUL, torch.bfloat16, 512, 4096, 1024, 0, 8) == (128 * 2 * 131072 + 65536, 2)
+    assert ops.kslice_plan(L.MATMUL_ALLREDUCE, torch.float16, 512, 1024, 1024, 0, 2) == (16 * 2 * 131072 + 65536, 2)
     assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 8192, 1792, 4096, 0, 8) == (0, 1)       # 1024 tiles
-    assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024, 4096, 1024, 0, 8) == (32 * 8 * 131072 + 256, 8)
+    assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024, 4096, 1024, 0, 8) == (32 * 8 * 131072 + 65536, 8)
     assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024, 4096, 1024, 0, 8, split_k=2)[1] == 2
     assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024 + 8, 4096, 1024, 0, 8) == (0, 1)   # ragged rows
     with pytest.raises(L.CatcocError, match="at most 2 k slices"):
         ops.kslice_plan(L.MATMUL_ALLREDUCE, torch.float16, 512, 1024, 1024, 0, 2, split_k=4)
     need, f, tiles = ops.splitk_plan(16, 8192, 8192, 8, 0, 2)
     assert (f, tiles) == (oracle.splitk_factor(16, 8192, 8192, 256, 128, 128, 256), 64)
-    assert need == f * tiles * 128 * 128 * 4 + 256
+    assert need == f * tiles * 128 * 128 * 4 + 65536    # counter block of a fixed size first, then the partial tiles
     need, f, tiles = ops.splitk_plan(512, 8192, 8192, 8, 0, 64)
     assert (need, f, tiles) == (0, 1, 256)
     need, f, tiles = ops.splitk_plan(200, 1088, 256, 4, 100, 50, split_k=3)
-    assert (f, tiles) == (3, 4) and need == 3 * 4 * 65536 + 256
+    assert (f, tiles) == (3, 4) and need == 3 * 4 * 65536 + 65536
     with pytest.raises(L.CatcocError, match="kept rows"):
         ops.splitk_plan(16, 8192, 8192, 8, 10, 7)
 
@@ -355,3 +355,72 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout == ""
+
+
+def test_python_entry_points_reject_mistyped_or_short_operands():
+    # The C ABI sees raw pointers, so element types and sizes are checked by the Python mirror before any launch;
+    # every rejection below is raised on host tensors, before the device check and without touching a GPU.
+    import torch
+    from mm_rs_with_catlass_amd import ops
+    M, K, N, P = 1024, 256, 512, 8
+    rows = M // P
+    x1 = torch.zeros((M, K), dtype=torch.int8)
+    x2 = torch.zeros((K, N), dtype=torch.int8)
+    s1 = torch.ones(M)
+    s2 = torch.ones(N)
+    peers = [torch.zeros((rows, N)) for _ in range(P - 1)]
+    q = ops.prepare_quant_matmul_reduce_scatter
+
+    def rejects(match, *a, **kw):
+        with pytest.raises(L.CatcocError, match=match):
+            q(*a, **kw)
+
+    rejects("x1 must be", x1.float(), x2, s1, s2, None, peers, 0, P)
+    rejects("scale_x1 must be", x1, x2, s1.half(), s2, None, peers, 0, P)
+    rejects("scale_x2 holds", x1, x2, s1, s2[:N - 1], None, peers, 0, P)
+    rejects("bias must be", x1, x2, s1, s2, torch.zeros(N), peers, 0, P)
+    rejects("k extent", x1, torch.zeros((K + 64, N), dtype=torch.int8), s1, s2, None, peers, 0, P)
+    rejects("k extent", x1, x2, s1, s2, None, peers, 0, P, trans_b=True)
+    rejects("rank_size - 1", x1, x2, s1, s2, None, peers[:-1], 0, P)
+    rejects(r"peers\[6\] has shape", x1, x2, s1, s2, None, peers[:-1] + [torch.zeros((rows - 1, N))], 0, P)
+    rejects(r"peers\[0\] has shape", x1, x2, s1, s2, None, peers, 0, P, peer_row_offset=1)
+    rejects(r"peers\[2\] must be", x1, x2, s1, s2, None, peers[:2] + [peers[2].int()] + peers[3:], 0, P)
+    rejects(r"peers\[0\] must be", x1, x2, s1, s2, None, peers, 0, P, reduce_int32=True)
+    rejects("m % rank_size", x1[:1020], x2, s1, s2, None, peers, 0, P)
+    rejects("out of range", x1, x2, s1, s2, None, peers, 8, P)
+    rejects("out must have shape", x1, x2, s1, s2, None, peers, 0, P, out=torch.zeros((rows, N - 1), dtype=torch.bfloat16))
+    rejects("out must be", x1, x2, s1, s2, None, peers, 0, P, out=torch.zeros((rows, N)))
+    rejects("c_accum holds", x1, x2, s1, s2, None, peers, 0, P, c_accum=torch.zeros((rows - 1, N), dtype=torch.int32))
+    rejects("acc_dump must be", x1, x2, s1, s2, None, peers, 0, P, acc_dump=torch.zeros((M, N)))
+    rejects("checksum holds", x1, x2, s1, s2, None, peers, 0, P, checksum=torch.zeros(15, dtype=torch.int64))   # 16 tasks
+    rejects("tiling says", x1, x2, s1, s2, None, peers, 0, P, tiling=ops.default_tiling(M, K, N + 256, P))
+    rejects("must live on the GPU", x1, x2, s1, s2, None, peers, 0, P)          # everything else in order: only the device is wrong
+
+    sk = ops.prepare_quant_matmul_splitk
+    a1 = torch.zeros((16, 256), dtype=torch.int8)
+    b1 = torch.zeros((256, 256), dtype=torch.int8)
+    with pytest.raises(L.CatcocError, match="kept rows"):
+        sk(a1, b1, torch.ones(16), torch.ones(256), None, [], 1, 10, 7)
+    with pytest.raises(L.CatcocError, match=r"peers\[0\] has shape"):
+        sk(a1, b1, torch.ones(16), torch.ones(256), None, [torch.zeros((1, 256))], 2, 0, 2)
+    with pytest.raises(L.CatcocError, match="checksum holds"):
+        sk(a1, b1, torch.ones(16), torch.ones(256), None, [], 1, 0, 2, checksum=torch.zeros(1, dtype=torch.int64))
+    with pytest.raises(L.CatcocError, match="scale_x1 holds"):
+        sk(a1, b1, torch.ones(15), torch.ones(256), None, [], 1, 0, 2)
+
+    a = torch.zeros((M, K), dtype=torch.float16)
+    b = torch.zeros((K, N), dtype=torch.float16)
+    with pytest.raises(L.CatcocError, match="both be float16 or both bfloat16"):
+        ops.matmul_reduce_scatter(a, b.bfloat16(), peers, 0, P)
+    with pytest.raises(L.CatcocError, match=r"peers\[0\] has shape"):
+        ops.matmul_allreduce(a, b, [torch.zeros((rows, N))], 0, 2)          # all-reduce peers are full [m,n]
+    with pytest.raises(L.CatcocError, match="k extent"):
+        ops.matmul_reduce_scatter(a, b, peers, 0, P, trans_a=True)
+    with pytest.raises(L.CatcocError, match=r"peer_shards\[0\] has shape"):
+        ops.allgather_matmul(a, [torch.zeros((M - 1, K), dtype=torch.float16)], b, 0, 2)
+    with pytest.raises(L.CatcocError, match=r"peer_shards\[0\] must be"):
+        ops.allgather_matmul(a, [torch.zeros((M, K))], b, 0, 2)
+    with pytest.raises(L.CatcocError, match="acc_dump holds"):
+        ops.allgather_matmul(a, [a.clone()], b, 0, 2, acc_dump=torch.zeros((M, N)))      # the gathered product has 2M rows
+    with pytest.raises(L.CatcocError, match="must live on the GPU"):
+        ops.matmul_reduce_scatter(a, b, peers, 0, P)

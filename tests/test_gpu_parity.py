@@ -87,7 +87,7 @@ def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, tran
     if kslices is not None:      # (forced count or 0 = the library's choice, count expected)
         need, f = ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, M, K, N, rank, P, tiling=tiling, split_k=kslices[0])
         assert f == kslices[1]
-        assert need == (ntasks * f * 128 * 256 * 4 + -(-ntasks * 4 // 256) * 256 if f > 1 else 0)
+        assert need == (ntasks * f * 128 * 256 * 4 + 65536 if f > 1 else 0)
         if f > 1:
             ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
             kw["workspace"] = ws
@@ -101,7 +101,7 @@ def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, tran
         if it + 1 < launches:
             out.zero_()
     if ws is not None:
-        assert not ws[ntasks * kslices[1] * 128 * 256 * 4:].any(), "tile counters were not re-armed"
+        assert not ws[:65536].any(), "tile counters were not re-armed"
     acc_got = acc_dump.cpu().numpy()
     assert np.array_equal(acc_got, acc_want), "int32 accumulators differ from the oracle"
     kept = acc_want[rank * rows:(rank + 1) * rows]
@@ -204,6 +204,51 @@ def test_quant_rs_few_tiles_k_sliced(case):
         if tr.value != rank:
             blk = r["acc"][row.value:row.value + 128, col.value:col.value + 256].astype(np.int64)
             assert cs[task] == blk.sum(), task
+
+
+def test_one_workspace_shared_by_launches_of_different_shapes():
+    # The arrival counters sit in a block of fixed size at the start of the workspace, so a workspace zeroed once serves
+    # launches of different tile counts and slice counts, k-sliced large tiles and skinny-M split-K alike, in any order.
+    _need_gpu()
+    rng = np.random.default_rng(77)
+    ws = torch.zeros(96 << 20, dtype=torch.uint8, device=DEV)
+
+    def ksliced(M, N, K, P, rank):
+        x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+        x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+        s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+        s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+        rows = M // P
+        peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+        _, want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, rank * rows, rows, peers, oracle.BF16, want_acc=False)
+        need, f = ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, M, K, N, rank, P)
+        assert f > 1 and need <= ws.numel()
+        out = ops.quant_matmul_reduce_scatter(dev(x1), dev(x2), dev(s1), dev(s2), None, [dev(p) for p in peers], rank, P, workspace=ws)
+        torch.cuda.synchronize()
+        assert np.array_equal(host16(out), want), (M, N, K)
+        return f
+
+    def skinny(M, N, K, P, kr):
+        x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+        x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+        s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+        s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+        peers = [rng.standard_normal((kr, N)).astype(np.float32) for _ in range(P - 1)]
+        _, want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, 0, kr, peers, oracle.BF16, want_acc=False)
+        need, f, tiles = ops.splitk_plan(M, K, N, P, 0, kr)
+        assert f > 1 and need <= ws.numel()
+        out = ops.quant_matmul_splitk(dev(x1), dev(x2), dev(s1), dev(s2), None, [dev(p) for p in peers], P, 0, kr, workspace=ws)
+        torch.cuda.synchronize()
+        assert np.array_equal(host16(out), want), (M, N, K)
+        return f
+
+    fs = [ksliced(1024, 1024, 4096, 4, 1),      # 32 tiles x 8 slices
+          skinny(16, 1024, 4096, 8, 2),         # 8 tiles of 128x128, split-K
+          ksliced(2048, 512, 1792, 8, 7),       # 32 tiles x 2 slices: counters where the first launch had partials
+          skinny(64, 2048, 2048, 4, 16),
+          ksliced(1024, 1024, 4096, 4, 2)]
+    assert fs[0] == 8 and fs[2] == 2
+    assert not ws[:65536].any(), "tile counters were not re-armed"
 
 
 def test_quant_rs_few_tiles_k_sliced_outbound_store():
@@ -323,6 +368,26 @@ def test_quant_rs_checksum_and_outbound_tiles():
         want = deq[row.value:row.value + m0, col.value:col.value + 256]
         assert np.array_equal(ob[ws.value:ws.value + m0].view(np.uint32), want.view(np.uint32)), task
 
+
+def test_quant_checksum_with_most_negative_operands_and_long_k():
+    # int8 admits -128: accumulators reach 128*128*k, and the checksum's 32-bit partial sums must still hold them
+    _need_gpu()
+    M, N, K, P, rank = 256, 256, 32704, 2, 1
+    x1 = torch.full((M, K), -128, dtype=torch.int8, device=DEV)
+    x2 = torch.full((K, N), -128, dtype=torch.int8, device=DEV)
+    s1 = torch.full((M,), 2.0 ** -20, device=DEV)
+    s2 = torch.full((N,), 2.0 ** -10, device=DEV)
+    peers = [torch.zeros((M // P, N), device=DEV)]
+    cs = torch.zeros(2, dtype=torch.int64, device=DEV)
+    dump = torch.zeros((M, N), dtype=torch.int32, device=DEV)
+    out = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, rank, P, checksum=cs, acc_dump=dump)
+    torch.cuda.synchronize()
+    acc = 128 * 128 * K
+    assert acc < 2 ** 31 and 4 * acc < 2 ** 31
+    assert torch.all(dump == acc)
+    assert sorted(cs.tolist()) == [0, 128 * 256 * acc]
+    want = torch.tensor(float(acc) * 2.0 ** -30).to(torch.bfloat16)     # power-of-two scales: only the final cast rounds
+    assert torch.all(out == want.to(DEV))
 
 def test_quant_fixed_config_entry_point():
     # catcoc_quant_matmul_reduce_scatter: the example's signature (m, n, k by value, bf16 out, tile 128x256,
@@ -614,6 +679,81 @@ def test_quant_config4_full_size_properties():
     assert torch.equal(out0.view(torch.int16), want0.view(torch.int16))
 
 
+def test_float_config3_full_size_properties():
+    """fp16 matmul-reduce-scatter benchmark config (A[4096,1792] N(0,1), B[1792,4096] N(0,0.02), P=8, 7 fp32 peers,
+    kept block [512,4096]) at full size: 512 tiles of 128x256, the launch order of the many-tile regime.  A row sample
+    of the kept block against the oracle; the whole local partial through row / column sums against fp64 GEMVs; the
+    other ranks' tiles through their per-task checksums."""
+    _need_gpu()
+    import ctypes as C
+    M, N, K, P, rank = 4096, 4096, 1792, 8, 5
+    g = torch.Generator(device=DEV).manual_seed(33)
+    A = torch.randn((M, K), device=DEV, generator=g).half()
+    B = (torch.randn((K, N), device=DEV, generator=g) * 0.02).half()
+    rows = M // P
+    peers = [torch.randn((rows, N), device=DEV, generator=g) for _ in range(P - 1)]
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    so = L.load()
+    ntasks = so.catcoc_get_task_count(L.MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+    assert ntasks == 512
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    cs = torch.zeros(ntasks, dtype=torch.float64, device=DEV)
+    out = ops.matmul_reduce_scatter(A, B, peers, rank, P, acc_dump=dump, checksum=cs)
+    torch.cuda.synchronize()
+    Ad, Bd = A.double(), B.double()
+    # sum_j C[i,j] = A[i,:] . rowsum(B); |C| ~ 0.85, fp32 accumulation error of a 1792-term dot ~1e-5 per element
+    want_rows = Ad @ Bd.sum(1)
+    assert (dump.double().sum(1) - want_rows).abs().max().item() <= 2e-2
+    want_cols = Ad.sum(0) @ Bd
+    assert (dump.double().sum(0) - want_cols).abs().max().item() <= 2e-2
+    # oracle on a row sample of the kept block
+    sel = np.arange(rank * rows, (rank + 1) * rows, 29)
+    part, want = oracle.matmul_reduce(host16(A[sel]), host16(B), oracle.FP16, 0, len(sel),
+                                      [p[sel - rank * rows].cpu().numpy() for p in peers], want_partial=True)
+    full = part + sum(p[sel - rank * rows].cpu().numpy() for p in peers)
+    _check_float(host16(out[sel - rank * rows]), want, full, oracle.FP16, K)
+    assert (ulp_diff16(host16(out[sel - rank * rows]), want) <= 1).mean() > 0.999
+    assert np.abs(dump[sel].cpu().numpy() - part).max() <= 1e-3
+    # every task of another rank left the sum of its tile; kept tasks leave their slot untouched
+    csh = cs.cpu().numpy()
+    tile_sums = dump.double().view(M // 128, 128, N // 256, 256).sum((1, 3)).cpu().numpy()
+    tr, row, col, ws = (C.c_uint32() for _ in range(4))
+    for task in range(ntasks):
+        assert so.catcoc_task_tile(L.MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row), C.byref(col), C.byref(ws))
+        want_cs = 0.0 if tr.value == rank else tile_sums[row.value // 128, col.value // 256]
+        assert abs(csh[task] - want_cs) <= 1e-6 * 128 * 256, task
+
+
+@pytest.mark.parametrize("M", [1, 16, 64, 128, 512])
+def test_quant_config5_full_size(M):
+    """W8A8 decode sweep config at full size (K = N = 8192, P = 8, rank 0 keeps rows [0, ceil(M/8))): kept rows bit
+    for bit against the oracle, the full int32 accumulators through exact row / column sums."""
+    _need_gpu()
+    K = N = 8192
+    P = 8
+    kr = -(-M // P)
+    g = torch.Generator(device=DEV).manual_seed(500 + M)
+    x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
+    x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=DEV, generator=g)
+    s1 = torch.empty(M, device=DEV).uniform_(0.005, 0.02, generator=g)
+    s2 = torch.empty(N, device=DEV).uniform_(0.001, 0.01, generator=g)
+    peers = [torch.randn((kr, N), device=DEV, generator=g) for _ in range(P - 1)]
+    need, f, tiles = ops.splitk_plan(M, K, N, P, 0, kr)
+    ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=DEV)
+    dump = torch.zeros((M, N), dtype=torch.int32, device=DEV)
+    out = ops.quant_matmul_splitk(x1, x2, s1, s2, None, peers, P, 0, kr, workspace=ws, acc_dump=dump)
+    torch.cuda.synchronize()
+    want_rows = x1.double() @ x2.double().sum(1)          # exact: every partial sum is an integer below 2^53
+    assert torch.equal(dump.to(torch.int64).sum(1), want_rows.to(torch.int64))
+    want_cols = x1.double().sum(0) @ x2.double()
+    assert torch.equal(dump.to(torch.int64).sum(0), want_cols.to(torch.int64))
+    acc_k, want = oracle.quant_matmul_reduce_scatter(x1[:kr].cpu().numpy(), x2.cpu().numpy(), s1[:kr].cpu().numpy(),
+                                                     s2.cpu().numpy(), None, 0, kr, [p.cpu().numpy() for p in peers], oracle.BF16)
+    assert np.array_equal(dump[:kr].cpu().numpy(), acc_k)
+    assert np.array_equal(host16(out), want), "kept rows differ from the oracle"
+
+
 # ------------------------------------------------------- C ABI from a plain C++ host
 def test_launches_replay_from_a_hip_graph():
     # serving loops capture their launches: the library allocates nothing and never synchronises, the split-K path
@@ -656,7 +796,7 @@ def test_launches_replay_from_a_hip_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out_big, want_big) and torch.equal(out_small, want_small)
-        assert not ws[tiles * fac * 128 * 128 * 4:].any(), "tile counters were not re-armed"
+        assert not ws[:65536].any(), "tile counters were not re-armed"
 
 
 def test_cpp_host_drives_the_library_through_the_c_abi(tmp_path):
@@ -699,7 +839,7 @@ def test_bench_prints_one_json_line_with_roofline():
     import subprocess
     import sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "3", "--warmup", "1", "--no-cpu"],
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "3", "--warmup", "1", "--no-cpu", "--sustained", "40"],
                        capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
@@ -713,3 +853,6 @@ def test_bench_prints_one_json_line_with_roofline():
     rf = d["roofline"]
     assert rf["bound"] == "mfma" and rf["peak"] == 5000.0 and abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3
     assert 100.0 < d["value"] < 5000.0
+    assert rf["kernel_us_sustained"] > 0 and len(rf["sustained_series_us"]) == 10 and rf["kernel_us_avg_same_buffers"] > 0
+    ob = d["outbound"]          # the reference's store mode rides along as a secondary object
+    assert ob["kept_block_equals_main_mode"] is True and ob["TOPS"] > 100.0 and ob["algorithmic_bytes"] > rf["algorithmic_bytes"]
