@@ -189,6 +189,21 @@ CATCOC_API void catcoc_launch_quant_matmul_reduce_scatter(void *stream, uint64_t
     uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum, uint8_t *d_out, uint8_t *symmetricPtr,
     CocTilingParams *tiling, uint32_t transA, uint32_t transB, uint32_t outDataType);
 
+/* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Arguments and results are exactly those
+ * of catcoc_launch_quant_matmul_reduce_scatter, except that desc->workspace / workspaceBytes are ignored: launches that
+ * cut their k range into slices (the skinny-M split-K path; few-tile launches of the large-tile kernel) meet through a
+ * scratch array built into the library, CATCOC_STATIC_SCRATCH_BYTES per GPU, which each GPU the library runs on holds
+ * until the process ends.  The call allocates nothing.  A launch that needs more scratch than that is rejected
+ * (catcoc_last_error() says how much it needs).  All calls on one GPU share that GPU's array: calls that overlap on
+ * one GPU (different streams, no ordering between them) race; calls on one stream, or ordered by events, are fine.
+ * The first call on a GPU also queues a small kernel on `stream` that zeroes the array's counter block; afterwards
+ * every launch leaves the counters at zero for the next. */
+#define CATCOC_STATIC_SCRATCH_BYTES (CATCOC_WORKSPACE_COUNTER_BYTES + (32u << 20))
+CATCOC_API void catcoc_launch_quant_matmul_reduce_scatter_static_scratch(void *stream, uint64_t fftsAddr, uint8_t *x1,
+    uint8_t *x2, uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum, uint8_t *d_out,
+    uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA, uint32_t transB, uint32_t outDataType);
+
 /* ----------------------------------------------------------------------- */
 /* Validation, errors, sizes                                                 */
 /* ----------------------------------------------------------------------- */

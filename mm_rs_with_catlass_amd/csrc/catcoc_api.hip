@@ -2,6 +2,7 @@
 // to the fused GEMM kernels.  Declarations and the reference interfaces they
 // replace are in include/catcoc_hip.h.
 #include <hip/hip_runtime.h>
+#include <pthread.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -403,9 +404,108 @@ void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uin
     ok();
 }
 
+// ---- built-in scratch for callers that cannot allocate ---------------------------------------
+// One array per GPU, part of the library's code object: it exists from the moment the library is loaded on a device
+// until the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress; everything that
+// needs the memory (kernel arguments, the fill below) uses the per-device address obtained from it.
+static __device__ __align__(256) unsigned char scratch[CATCOC_STATIC_SCRATCH_BYTES];
+
+__global__ void scratch_zero_kernel(uint32_t *p, uint32_t words)
+{
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x) p[i] = 0u;
+}
+
+constexpr int kMaxDevices = 64;
+struct ScratchState { void *ptr; bool cleared; };
+ScratchState g_scratch[kMaxDevices];
+pthread_mutex_t g_scratchLock = PTHREAD_MUTEX_INITIALIZER;
+
+// Address of the current device's copy of `scratch`; on the first call on a device also queues, on `stream`, a kernel
+// that zeroes the counter block (a kernel, not a memset: the call may be under stream capture).  NULL on failure.
+void *scratch_for_current_device(void *stream)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        fail(E_LAUNCH, "no current HIP device (or more than %d devices)", kMaxDevices);
+        return nullptr;
+    }
+    pthread_mutex_lock(&g_scratchLock);
+    ScratchState &st = g_scratch[dev];
+    if (st.ptr == nullptr) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            pthread_mutex_unlock(&g_scratchLock);
+            fail(E_LAUNCH, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        st.ptr = p;
+    }
+    if (!st.cleared) {
+        hipLaunchKernelGGL(scratch_zero_kernel, dim3(16), dim3(256), 0, (hipStream_t)stream, (uint32_t *)st.ptr,
+                           (uint32_t)(kCounterBlockBytes / 4u));
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            pthread_mutex_unlock(&g_scratchLock);
+            fail(E_LAUNCH, "clearing the built-in scratch failed: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        st.cleared = true;
+    }
+    void *p = st.ptr;
+    pthread_mutex_unlock(&g_scratchLock);
+    return p;
+}
+
 }  // namespace
 
 extern "C" {
+
+void catcoc_launch_quant_matmul_reduce_scatter_static_scratch(void *stream, uint64_t fftsAddr, uint8_t *x1, uint8_t *x2,
+                                                              uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias,
+                                                              uint8_t *c_accum, uint8_t *d_out, uint8_t *symmetricPtr,
+                                                              CocTilingParams *tiling, uint32_t transA, uint32_t transB,
+                                                              uint32_t outDataType)
+{
+    (void)fftsAddr;
+    const CatcocSymmetricDesc *given = (const CatcocSymmetricDesc *)symmetricPtr;
+    if (given == nullptr || given->magic != CATCOC_DESC_MAGIC) {
+        fail(E_DESC, "symmetricPtr does not point at a CatcocSymmetricDesc");
+        return;
+    }
+    CatcocSymmetricDesc d = *given;
+    d.workspace = nullptr;
+    d.workspaceBytes = 0;
+    // how much scratch would this launch use?  Plan it first, with the sizes only.
+    uint64_t need = 0;
+    {
+        CatcocSymmetricDesc q = d;
+        for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!q.peers[i]) q.peers[i] = (const void *)16;
+        if (q.keptRows != 0) {
+            SplitkPlan sp;
+            if (make_splitk_plan(tiling, &q, transA, transB, sp)) return;
+            need = sp.workspaceBytes;
+        } else {
+            Plan p;
+            q.flags &= ~CATCOC_OUTBOUND_MASK;
+            if (make_plan(QUANT_MATMUL_REDUCE_SCATTER, INT8, tiling, &q, transA, transB, p)) return;
+            need = p.kSliceBytes;
+        }
+    }
+    if (need > (uint64_t)CATCOC_STATIC_SCRATCH_BYTES) {
+        fail(E_WORKSPACE, "this launch needs %llu bytes of scratch; the built-in scratch holds %llu "
+                          "(use catcoc_launch_quant_matmul_reduce_scatter with a workspace of your own)",
+             (unsigned long long)need, (unsigned long long)CATCOC_STATIC_SCRATCH_BYTES);
+        return;
+    }
+    if (need != 0) {
+        void *p = scratch_for_current_device(stream);
+        if (p == nullptr) return;
+        d.workspace = p;
+        d.workspaceBytes = CATCOC_STATIC_SCRATCH_BYTES;
+    }
+    launch_quant(stream, x1, x2, scale_x1, scale_x2, bias, c_accum, d_out, (uint8_t *)&d, tiling, transA, transB, outDataType);
+}
 
 #define FLOAT_LAUNCHER(name, commType, dataType)                                                                      \
     void name(void *stream, uint64_t fftsAddr, uint8_t *a, uint8_t *b, uint8_t *c, uint8_t *aW, uint8_t *bW,           \

@@ -16,6 +16,7 @@ BF16 = 27
 
 MAX_RANKS = 16
 WORKSPACE_COUNTER_BYTES = 65536
+STATIC_SCRATCH_BYTES = WORKSPACE_COUNTER_BYTES + (32 << 20)
 DESC_MAGIC = 0x43544343
 OUTBOUND_CHECKSUM = 0
 OUTBOUND_STORE = 1
@@ -60,6 +61,7 @@ EXPORTS = [
     "catcoc_launch_allgather_matmul_fp16", "catcoc_launch_allgather_matmul_bf16",
     "catcoc_launch_matmul_reduce_scatter_fp16", "catcoc_launch_matmul_reduce_scatter_bf16",
     "catcoc_quant_matmul_reduce_scatter", "catcoc_launch_quant_matmul_reduce_scatter",
+    "catcoc_launch_quant_matmul_reduce_scatter_static_scratch",
     "catcoc_last_error", "catcoc_last_status", "catcoc_can_implement", "catcoc_get_workspace_size",
     "catcoc_get_splitk_workspace_size", "catcoc_get_kslice_workspace_size",
     "catcoc_get_task_count", "catcoc_get_tilings", "catcoc_check_comm_interval_reduce_scatter",
@@ -119,6 +121,8 @@ def load():
     L.catcoc_launch_quant_matmul_reduce_scatter.argtypes = [vp, C.c_uint64] + [vp] * 8 + [
         C.POINTER(CocTilingParams), u32, u32, u32]
     L.catcoc_launch_quant_matmul_reduce_scatter.restype = None
+    L.catcoc_launch_quant_matmul_reduce_scatter_static_scratch.argtypes = L.catcoc_launch_quant_matmul_reduce_scatter.argtypes
+    L.catcoc_launch_quant_matmul_reduce_scatter_static_scratch.restype = None
     L.catcoc_last_error.restype = C.c_char_p
     L.catcoc_last_status.restype = C.c_int
     L.catcoc_can_implement.argtypes = [C.c_int, C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32, u32]
