@@ -205,6 +205,49 @@ CATCOC_API void catcoc_launch_quant_matmul_reduce_scatter_static_scratch(void *s
     uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA, uint32_t transB, uint32_t outDataType);
 
 /* ----------------------------------------------------------------------- */
+/* Round-pipelined, reference-faithful form                                  */
+/* ----------------------------------------------------------------------- */
+
+/* The reduce-scatter operators with the reference's own structure instead of the fused epilogue
+ * (include/catcoc/dgemm/kernel/quant_matmul_reduce_scatter.hpp:159-164,219,282,319 and matmul_reduce_scatter.hpp:155-199,
+ * 237-296): comm rounds of blockNum x commInterval tiles; per round the GEMM (on computeStream) stores the round's tiles --
+ * the kept rank's into the local block, the others into stage `round % workspaceStages` of desc->outbound in the
+ * tile-linear layout -- then the comm side (on commStream) adds the peers' blocks into the local block along
+ * BlockCommSwizzle's task list; the GEMM of round + workspaceStages waits for that before it reuses the stage.  The two
+ * cross-core flags per stage are HIP events between the two streams (created and destroyed inside the call); on return
+ * computeStream is ordered after the finished output.  commBlockM (0 = 64) must divide m0; commDataSplit x commNpuSplit
+ * is the number of comm "cores" (workgroups), raised to 256 x 1 when below 16.
+ *   W8A8: int32 tiles; peers[] are int32 partials [m/P, n] added into c_accum (required, receives the reduced int32
+ *   block) with integer adds, then one dequant pass writes d_out (quant_matmul_reduce_scatter.hpp:285-351).  Bit-identical
+ *   to catcoc_launch_quant_matmul_reduce_scatter with CATCOC_FLAG_REDUCE_INT32.
+ *   fp16 / bf16: the local partial is rounded to the output type and peers[] are 16-bit partials [m/P, n] of that type,
+ *   each added with one rounding to that type (matmul_reduce_scatter.hpp:261; the fp32 -> 16-bit cast of
+ *   3rdparty/catlass/include/catlass/gemm/tile/copy_l0c_to_gm.hpp:39-57).
+ * deterministic != 0 runs BlockCommSwizzle<0, true> (comm_block_swizzle.hpp:25-31,54-56,114-118): one core owns a data
+ * block and adds the ranks in the order (dataIdx + i) % rankSize, so 16-bit results are reproducible; 0 runs
+ * BlockCommSwizzle<0, false> with hardware atomic adds in arrival order, like the reference. */
+CATCOC_API void catcoc_pipelined_quant_matmul_reduce_scatter(void *computeStream, void *commStream, uint64_t fftsAddr,
+    uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum, uint8_t *d_out,
+    uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA, uint32_t transB, uint32_t outDataType,
+    uint32_t deterministic);
+CATCOC_API void catcoc_pipelined_matmul_reduce_scatter(void *computeStream, void *commStream, int dataType, uint8_t *a,
+    uint8_t *b, uint8_t *c, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA, uint32_t transB,
+    uint32_t deterministic);
+
+/* SplitkMatmul's ReduceAdd as a kernel of its own (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:24-161):
+ * src holds splitkFactor fp32 slices of elementCount elements each, back to back; dst[i] = the slices' sum in slice order
+ * (fp32 adds), rounded once to outDataType (FP16 / BF16, or 0 to keep fp32).  16-byte aligned buffers. */
+CATCOC_API void catcoc_reduce_add(void *stream, uint8_t *dst, uint8_t *src, uint64_t elementCount, uint32_t splitkFactor,
+                                  uint32_t outDataType);
+
+/* The reference's accuracy gate (examples/utils/verify_result.py:26-43,88-117 with the tolerances of
+ * examples/utils/utils.py:44-52) on host arrays: every element |out - gold| <= rtol * max(1, |gold|) with
+ * rtol = 2^-8 (fp16) / 2^-7 (bf16) for computeTimes < 2048 and twice that otherwise, and
+ * |mean((out - gold) / max(1, |gold|))| <= 2^-10 (fp16) / 2^-7 (bf16); NaN and Inf count as 0.  Returns 1 on pass. */
+CATCOC_API int catcoc_verify(const float *out, const float *gold, uint64_t count, int dataType, uint32_t computeTimes,
+                             uint64_t *nBad, double *meanRelErr);
+
+/* ----------------------------------------------------------------------- */
 /* Validation, errors, sizes                                                 */
 /* ----------------------------------------------------------------------- */
 
@@ -293,6 +336,14 @@ CATCOC_API void catcoc_allgather_block_coord(uint32_t off, uint32_t dir, uint32_
 CATCOC_API void catcoc_comm_block_idx(uint32_t dir, uint32_t P, uint32_t splitRow, uint32_t splitCol,
                                       uint32_t dataLoopsInRank, uint32_t task, uint32_t *dataIdx,
                                       uint32_t *rankIdx);
+/* BlockCommSwizzle<dir, deterministic>::GetBlockIdx / GetCoreLoop (comm_block_swizzle.hpp:25-31,54-56,106-118,147-186).
+ * With deterministic != 0 (direction 0 only) the npu split folds into the data split and the last band is padded:
+ * data indices >= dataLoopsInRank are padding tasks. */
+CATCOC_API void catcoc_comm_block_idx_ex(uint32_t dir, uint32_t deterministic, uint32_t P, uint32_t splitRow,
+                                         uint32_t splitCol, uint32_t dataLoopsInRank, uint32_t task, uint32_t *dataIdx,
+                                         uint32_t *rankIdx);
+CATCOC_API uint32_t catcoc_comm_core_loop(uint32_t deterministic, uint32_t P, uint32_t splitRow, uint32_t splitCol,
+                                          uint32_t dataLoopsInRank);
 /* The tile a task computes in each operator (quant_matmul_reduce_scatter.hpp:172-201,
  * matmul_allreduce.hpp:154-179, allgather_matmul.hpp:142-163): target rank, first row/col of the tile in
  * the global problem, and the workspace row of the reference's tile-linear layout.  Returns 0 past the end. */

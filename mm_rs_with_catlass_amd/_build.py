@@ -8,6 +8,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
 LIB = os.path.join(PKG, "libcatcoc_hip.so")
 HOST_EXAMPLE = os.path.join(PKG, "catcoc_quant_rs_host")   # C++ host driving the library through its C ABI alone
+FACADE_EXAMPLE = os.path.join(PKG, "catcoc_facade_host")  # C++ host written against the template facade (catcoc_hip/dgemm.hpp)
 OBJ_DIR = os.path.join(PKG, "csrc", "build")
 
 HIPCC_FLAGS = [
@@ -54,6 +55,13 @@ def build(verbose=False, extra=(), jobs=8):
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     cmd = [cxx, "-O2", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"), "-I", os.path.join(rocm, "include"),
            os.path.join(PKG, "csrc", "host_quant_rs.cpp"), "-o", HOST_EXAMPLE, "-L", PKG, "-lcatcoc_hip",
+           "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    # the host written against the reference's kernel-template names (include/catcoc_hip/dgemm.hpp), also plain g++
+    cmd = [cxx, "-O2", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(ROOT, "include"), "-I", os.path.join(rocm, "include"),
+           os.path.join(PKG, "csrc", "host_facade.cpp"), "-o", FACADE_EXAMPLE, "-L", PKG, "-lcatcoc_hip",
            "-L", os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(rocm, "lib")]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -7,7 +7,12 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <math.h>
+
+#include <vector>
+
 #include "catcoc_hip.h"
+#include "comm_reduce.h"
 #include "gemm_args.h"
 #include "tile_sched.h"
 
@@ -401,6 +406,125 @@ void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uin
     if (!dma) p.args.splitK = 0;   // the other kernels run every tile whole
     const int e = dma ? launch_gemm_dma_i8(p.args, stream) : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
+    ok();
+}
+
+// ---- round-pipelined, reference-faithful form of the reduce-scatter operators ------------------
+// The reference's structure kept as it is (quant_matmul_reduce_scatter.hpp:159-164,219,282,319; matmul_reduce_scatter.hpp
+// the same): per comm round the GEMM stores the round's tiles (kept rank's into the local block, the others into stage
+// `round % stages` of the workspace) and raises "store finished"; the comm side waits for it, adds the peers' blocks into
+// the local block along BlockCommSwizzle's task list and raises "compute finished", which the GEMM of round + stages
+// waits for before it reuses the stage.  The two sides are two HIP streams here and the flags are events.
+void launch_pipelined(bool quant, int dataType, void *computeStream, void *commStream, uint8_t *a, uint8_t *b, uint8_t *scale_x1,
+                      uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum, uint8_t *d_out, uint8_t *symmetricPtr,
+                      CocTilingParams *tiling, uint32_t transA, uint32_t transB, uint32_t outDataType, uint32_t deterministic)
+{
+    const CatcocSymmetricDesc *given = (const CatcocSymmetricDesc *)symmetricPtr;
+    if (given == nullptr || given->magic != CATCOC_DESC_MAGIC) { fail(E_DESC, "symmetricPtr does not point at a CatcocSymmetricDesc"); return; }
+    if (given->keptRows != 0) { fail(E_DESC, "the round-pipelined form keeps the reference's row blocks (keptRows must be 0)"); return; }
+    CatcocSymmetricDesc d = *given;
+    d.flags = (d.flags & ~CATCOC_OUTBOUND_MASK) | CATCOC_OUTBOUND_STORE | CATCOC_FLAG_LINEAR_ORDER;
+    if (quant) d.flags |= CATCOC_FLAG_REDUCE_INT32;
+    d.workspace = nullptr;
+    d.splitK = 0;
+    Plan p;
+    const int commType = quant ? QUANT_MATMUL_REDUCE_SCATTER : MATMUL_REDUCE_SCATTER;
+    if (make_plan(commType, dataType, tiling, &d, transA, transB, p)) return;
+    if (!a || !b || !d_out) { fail(E_NULL, "operands and output must be non-NULL"); return; }
+    if (quant && (!scale_x1 || !scale_x2 || !c_accum)) { fail(E_NULL, "the pipelined W8A8 operator needs scale_x1, scale_x2 and c_accum"); return; }
+    const uint32_t outDt = quant ? outDataType : (uint32_t)dataType;
+    if (outDt != FP16 && outDt != BF16) { fail(E_DTYPE, "outDataType %u must be FP16 (1) or BF16 (27)", outDt); return; }
+    if (d.outbound == nullptr && d.rankSize > 1) { fail(E_NULL, "the pipelined form stores the other ranks' tiles: outbound (the symmetric workspace) is needed"); return; }
+
+    GemmArgs &g = p.args;
+    const SchedParams &sp = g.sched;
+    const uint32_t P = sp.P, m0 = sp.m0, n0 = sp.n0;
+    const uint32_t cb = tiling->commBlockM ? tiling->commBlockM : umin(64u, m0);
+    if (m0 % cb != 0) { fail(E_TILING, "commBlockM %u must divide m0 %u", cb, m0); return; }
+    uint32_t splitRow = tiling->commDataSplit, splitCol = tiling->commNpuSplit ? tiling->commNpuSplit : 1u;
+    if (splitRow == 0 || splitRow * splitCol < 16u) { splitRow = 256u; splitCol = 1u; }   // the reference's 2..20 cores would idle this GPU
+    if (!deterministic && P % splitCol != 0) { fail(E_TILING, "commNpuSplit %u must divide rankSize %u", splitCol, P); return; }
+    const uint32_t es = quant ? 4u : 2u;
+    const uint32_t vec = 16u / es;
+    if (tiling->n % vec != 0 || n0 % vec != 0) { fail(E_SHAPE, "the pipelined form moves 16-byte pieces: n and n0 must be multiples of %u", vec); return; }
+    const int64_t peerLd = d.peerLd ? d.peerLd : tiling->n;
+    void *local = quant ? (void *)c_accum : (void *)d_out;
+    if ((uintptr_t)local % 16 != 0 || (peerLd * es) % 16 != 0) { fail(E_SHAPE, "the pipelined form needs 16-byte aligned blocks and peer rows"); return; }
+    for (uint32_t s = 0; s + 1 < P; ++s)
+        if ((uintptr_t)d.peers[s] % 16 != 0) { fail(E_SHAPE, "peers[%u] must be 16-byte aligned", s); return; }
+
+    // GEMM side: every round is one launch of the ordinary kernels over the round's tasks, with no peers to add
+    if (quant) {
+        g.a[0] = a; g.b = b; g.d = d_out;
+        g.scaleM = (const float *)scale_x1; g.scaleN = (const float *)scale_x2;
+        g.bias = (const int32_t *)bias; g.cAccum = (int32_t *)c_accum;
+        g.outDtype = outDt;
+        if (!check_ptr_align(p, a, b) || (uintptr_t)scale_x2 % 16 != 0 || (bias && (uintptr_t)bias % 16 != 0) || (uintptr_t)d_out % 8 != 0) p.variant = 0;
+    } else {
+        g.a[0] = a; g.b = b; g.d = d_out;
+        if (!check_ptr_align(p, a, b)) p.variant = 0;
+    }
+    g.nPeers = 0;
+    const bool dma = !quant && p.dma && p.variant != 0 && (uintptr_t)b % 16 == 0 && (g.ldb * 2) % 16 == 0 && (uintptr_t)d_out % 16 == 0;
+    if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles and 16-byte aligned row-major operands"); return; }
+
+    CommArgs c;
+    memset(&c, 0, sizeof(c));
+    c.local = local;
+    c.localLd = tiling->n;
+    for (uint32_t s = 0; s + 1 < P; ++s) c.peers[s] = d.peers[s];
+    c.peerLd = peerLd;
+    c.peerRowOffset = d.peerRowOffset;
+    c.P = P; c.rank = d.rankIdx;
+    c.mRank = sp.mRank; c.N = tiling->n;
+    c.m0 = m0; c.n0 = n0; c.loopsM = sp.loopsM; c.loopsN = sp.loopsN; c.off = sp.off; c.dir = sp.dir;
+    c.commBlockM = cb;
+    c.splitRow = splitRow; c.splitCol = splitCol;
+    c.swizzleDir = 0;
+    c.dtype = quant ? (uint32_t)CT_INT32 : outDt;
+    const uint32_t cores = splitRow * splitCol;
+
+    const uint32_t bpc = sp.blockPerComm, perRank = bpc / P, stages = sp.stages;
+    const uint32_t rounds = ceil_div(sp.coreLoops, bpc);
+    std::vector<hipEvent_t> ready(rounds), done(rounds);
+    hipEvent_t fin = nullptr;
+    auto destroy = [&]() {
+        for (hipEvent_t e : ready) if (e) (void)hipEventDestroy(e);
+        for (hipEvent_t e : done) if (e) (void)hipEventDestroy(e);
+        if (fin) (void)hipEventDestroy(fin);
+    };
+    for (uint32_t r = 0; r < rounds; ++r) ready[r] = done[r] = nullptr;
+    hipError_t he = hipEventCreateWithFlags(&fin, hipEventDisableTiming);
+    for (uint32_t r = 0; r < rounds && he == hipSuccess; ++r) {
+        he = hipEventCreateWithFlags(&ready[r], hipEventDisableTiming);
+        if (he == hipSuccess) he = hipEventCreateWithFlags(&done[r], hipEventDisableTiming);
+    }
+    if (he != hipSuccess) { destroy(); fail(E_LAUNCH, "hipEventCreate failed: %s", hipGetErrorString(he)); return; }
+    hipStream_t cs = (hipStream_t)computeStream, ms = (hipStream_t)commStream;
+    int e = 0;
+    for (uint32_t r = 0; r < rounds && e == 0 && he == hipSuccess; ++r) {
+        const uint32_t first = r * bpc, actual = umin(bpc, sp.coreLoops - first);
+        if (r >= stages) he = hipStreamWaitEvent(cs, done[r - stages], 0);        // "compute finished" of the stage's last user
+        g.taskBase = first;
+        g.taskCount = actual;
+        if (he == hipSuccess)
+            e = dma ? (p.dtype == DT_F16 ? launch_gemm_dma_f16(g, computeStream) : launch_gemm_dma_bf16(g, computeStream))
+                    : launch_gemm(p.dtype, g, p.variant, p.edge, computeStream);
+        if (e == 0 && he == hipSuccess) he = hipEventRecord(ready[r], cs);        // "store finished"
+        if (e == 0 && he == hipSuccess) he = hipStreamWaitEvent(ms, ready[r], 0);
+        c.roundFirstIdx = r * perRank;
+        c.dataLoops = (actual / P) * (m0 / cb);
+        if (e == 0 && he == hipSuccess && P > 1 && c.dataLoops > 0) e = launch_comm_reduce(c, cores, deterministic != 0, commStream);
+        if (e == 0 && he == hipSuccess) he = hipEventRecord(done[r], ms);
+    }
+    if (e == 0 && he == hipSuccess && quant)   // the pass after all rounds: dequantise the reduced int32 block
+        e = launch_dequant_rows((const int32_t *)c_accum, tiling->n, (const float *)scale_x2, (const float *)scale_x1 + (size_t)d.rankIdx * sp.mRank,
+                                d_out, tiling->n, sp.mRank, tiling->n, outDt, commStream);
+    if (e == 0 && he == hipSuccess) he = hipEventRecord(fin, ms);
+    if (e == 0 && he == hipSuccess) he = hipStreamWaitEvent(cs, fin, 0);           // the caller's stream sees the finished output
+    destroy();
+    if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
+    if (he != hipSuccess) { fail(E_LAUNCH, "stream/event call failed: %s", hipGetErrorString(he)); return; }
     ok();
 }
 
@@ -830,6 +954,75 @@ int catcoc_device_info(int *cuCount, int *clockMHz, char *name, int nameLen)
     return 0;
 }
 
-const char *catcoc_version(void) { return "catcoc-hip 0.1 (gfx950)"; }
+const char *catcoc_version(void) { return "catcoc-hip 0.2 (gfx950)"; }
+
+void catcoc_pipelined_quant_matmul_reduce_scatter(void *computeStream, void *commStream, uint64_t fftsAddr, uint8_t *x1, uint8_t *x2,
+                                                  uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum, uint8_t *d_out,
+                                                  uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA, uint32_t transB,
+                                                  uint32_t outDataType, uint32_t deterministic)
+{
+    (void)fftsAddr;
+    launch_pipelined(true, INT8, computeStream, commStream, x1, x2, scale_x1, scale_x2, bias, c_accum, d_out, symmetricPtr, tiling, transA,
+                     transB, outDataType, deterministic);
+}
+
+void catcoc_pipelined_matmul_reduce_scatter(void *computeStream, void *commStream, int dataType, uint8_t *a, uint8_t *b, uint8_t *c,
+                                            uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA, uint32_t transB,
+                                            uint32_t deterministic)
+{
+    launch_pipelined(false, dataType, computeStream, commStream, a, b, nullptr, nullptr, nullptr, nullptr, c, symmetricPtr, tiling, transA,
+                     transB, (uint32_t)dataType, deterministic);
+}
+
+void catcoc_reduce_add(void *stream, uint8_t *dst, uint8_t *src, uint64_t elementCount, uint32_t splitkFactor, uint32_t outDataType)
+{
+    if (!dst || !src) { fail(E_NULL, "dst and src must be non-NULL"); return; }
+    if (splitkFactor == 0) { fail(E_TILING, "splitkFactor must be at least 1"); return; }
+    if (outDataType != 0 && outDataType != FP16 && outDataType != BF16) { fail(E_DTYPE, "outDataType %u must be 0 (fp32), FP16 or BF16", outDataType); return; }
+    if (elementCount == 0) { ok(); return; }
+    if ((uintptr_t)src % 16 != 0 || (uintptr_t)dst % 16 != 0 || (splitkFactor > 1 && elementCount % 4 != 0)) {
+        fail(E_SHAPE, "reduce-add needs 16-byte aligned buffers and, with more than one slice, an element count that is a multiple of 4");
+        return;
+    }
+    const int e = launch_reduce_add(dst, (const float *)src, elementCount, splitkFactor, outDataType, stream);
+    if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
+    ok();
+}
+
+int catcoc_verify(const float *out, const float *gold, uint64_t count, int dataType, uint32_t computeTimes, uint64_t *nBad, double *meanRelErr)
+{
+    // examples/utils/utils.py:44-52 and verify_result.py:34-43,88-117
+    if ((!out || !gold) && count) { fail(E_NULL, "out and gold must be non-NULL"); return 0; }
+    if (dataType != FP16 && dataType != BF16) { fail(E_DTYPE, "dataType %d must be FP16 or BF16", dataType); return 0; }
+    const float rtol = dataType == FP16 ? (computeTimes < 2048 ? 1.0f / 256 : 1.0f / 128) : (computeTimes < 2048 ? 1.0f / 128 : 1.0f / 64);
+    const double meanLimit = dataType == FP16 ? 1.0 / 1024 : 1.0 / 128;
+    uint64_t bad = 0;
+    double sum = 0.0;
+    for (uint64_t i = 0; i < count; ++i) {
+        float o = out[i], g = gold[i];
+        if (isnan(o) || isinf(o)) o = 0.0f;       // NaN / Inf are zeroed before the comparison
+        if (isnan(g) || isinf(g)) g = 0.0f;
+        const float scale = fabsf(g) > 1.0f ? fabsf(g) : 1.0f;
+        const float diff = o - g;
+        if (fabsf(diff) - rtol * scale > 0.0f) ++bad;
+        sum += (double)(diff / scale);
+    }
+    const double mean = count ? fabs(sum / (double)count) : 0.0;
+    if (nBad) *nBad = bad;
+    if (meanRelErr) *meanRelErr = mean;
+    ok();
+    return bad == 0 && mean <= meanLimit;
+}
+
+void catcoc_comm_block_idx_ex(uint32_t dir, uint32_t deterministic, uint32_t P, uint32_t splitRow, uint32_t splitCol,
+                              uint32_t dataLoopsInRank, uint32_t task, uint32_t *dataIdx, uint32_t *rankIdx)
+{
+    comm_block_idx_ex(dir, deterministic != 0, P, splitRow, splitCol, dataLoopsInRank, task, *dataIdx, *rankIdx);
+}
+
+uint32_t catcoc_comm_core_loop(uint32_t deterministic, uint32_t P, uint32_t splitRow, uint32_t splitCol, uint32_t dataLoopsInRank)
+{
+    return comm_core_loop(deterministic != 0, P, splitRow, splitCol, dataLoopsInRank);
+}
 
 }  // extern "C"

@@ -38,11 +38,15 @@ struct GemmArgs {
     uint32_t flags;                // GF_*
     uint32_t outDtype;             // DT_F16 / DT_BF16
     uint32_t transA, transB;
+    uint32_t taskBase, taskCount;  // positions [taskBase, taskBase + taskCount) of the launch order (round-by-round launches); taskCount 0 = all
     // Skinny-M split-K launch: k slices per tile, int32 partial tiles [splitK][tiles][128][128], one counter per tile.
     uint32_t splitK;
     int32_t *skPart;
     uint32_t *skCount;
     SchedParams sched;
 };
+
+// Workgroups (before k slicing) a launch starts.
+inline uint32_t launch_positions(const GemmArgs &a) { return a.taskCount ? a.taskCount : a.sched.coreLoops; }
 
 }  // namespace catcoc

@@ -103,7 +103,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const bool linear = (args.flags & GF_LINEAR_ORDER) != 0;
     // A launch with few tiles can cut every tile's k range into kSlices pieces, one workgroup each (128-row tiles
     // only): position `pos` of the launch order runs as kSlices workgroups that stay in the position's XCD column.
-    uint32_t pos = blockIdx.x, slice = 0;
+    uint32_t pos = blockIdx.x + args.taskBase, slice = 0;   // (taskBase is zero for k-sliced launches)
     const uint32_t kSlices = (WM == 2 && args.splitK > 1) ? args.splitK : 1u;
     if (kSlices > 1) {
         if ((sp.coreLoops & 7u) == 0) {

@@ -122,7 +122,7 @@ __global__ void __launch_bounds__(256, (MB <= 2) ? 2 : 1) gemm_fused_kernel(cons
     const int c32 = lane & 31, h = lane >> 5;
 
     const SchedParams &sp = args.sched;
-    const uint32_t task = launch_order_task(sp, blockIdx.x, (args.flags & GF_LINEAR_ORDER) != 0, args.keptRank);
+    const uint32_t task = launch_order_task(sp, blockIdx.x + args.taskBase, (args.flags & GF_LINEAR_ORDER) != 0, args.keptRank);
     TileInfo ti;
     if (!task_tile(sp, task, ti)) return;
 
@@ -500,7 +500,7 @@ template <uint32_t DT>
 __global__ void __launch_bounds__(256) gemm_general_kernel(const GemmArgs args)
 {
     const SchedParams &sp = args.sched;
-    const uint32_t task = blockIdx.x;
+    const uint32_t task = blockIdx.x + args.taskBase;
     TileInfo ti;
     if (!task_tile(sp, task, ti)) return;
     const bool gather = sp.op == OP_ALLGATHER;
@@ -605,7 +605,7 @@ __global__ void __launch_bounds__(256) gemm_general_kernel(const GemmArgs args)
 template <uint32_t DT, int MB, bool TRANSB>
 static hipError_t launch_fast(const GemmArgs &args, bool edge, hipStream_t stream)
 {
-    const dim3 grid(args.sched.coreLoops), block(256);
+    const dim3 grid(launch_positions(args)), block(256);
     if (edge) hipLaunchKernelGGL((gemm_fused_kernel<DT, MB, TRANSB, true>), grid, block, 0, stream, args);
     else hipLaunchKernelGGL((gemm_fused_kernel<DT, MB, TRANSB, false>), grid, block, 0, stream, args);
     return hipGetLastError();
@@ -617,7 +617,7 @@ static int launch_dt(const GemmArgs &args, int variant, bool edge, void *stream)
 {
     hipStream_t s = (hipStream_t)stream;
     if (variant == 0) {
-        hipLaunchKernelGGL((gemm_general_kernel<DT>), dim3(args.sched.coreLoops), dim3(256), 0, s, args);
+        hipLaunchKernelGGL((gemm_general_kernel<DT>), dim3(launch_positions(args)), dim3(256), 0, s, args);
         return (int)hipGetLastError();
     }
     if (args.transB) {

@@ -13,12 +13,12 @@ int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream)
 int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
 {
     if (args.sched.m0 == 256)
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), dim3(args.sched.coreLoops), dim3(512), 0, (hipStream_t)stream, args);
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
     else if (args.transB)   // B as [n][k]
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true>), dim3(args.sched.coreLoops * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
                            (hipStream_t)stream, args);
     else   // one workgroup per tile, or per k slice of a tile
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2>), dim3(args.sched.coreLoops * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
                            (hipStream_t)stream, args);
     return (int)hipGetLastError();
 }

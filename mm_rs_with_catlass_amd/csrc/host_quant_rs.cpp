@@ -10,6 +10,8 @@
 //   <dir>/peer_<s>.bin     fp32  [m/rankSize, n], s = 0..rankSize-2: the other ranks' dequantised partials
 //                          for this rank's rows (what the SHMEM gets would have pulled)
 //   <dir>/output.bin       bf16  [m,n]: this rank's [m/rankSize, n] block is written at its offset
+//   <dir>/golden.bin       fp32  [m,n]  (optional): when present, this rank's rows are checked against it with the
+//                          reference's accuracy gate (examples/utils/verify_quant_result.py) and the exit code is 4 on failure
 //
 // usage: catcoc_quant_rs_host <rankSize> <rankId> <m> <n> <k> [dir=./output]
 #include <hip/hip_runtime_api.h>
@@ -17,6 +19,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <string>
 #include <vector>
 
@@ -126,10 +129,36 @@ int main(int argc, char **argv)
     }
     if (rankId == 0) std::printf("test finished\n");
 
+    // verify_quant_result.py's check, when the reference's golden.bin (fp32 [m,n]) sits next to the inputs: this rank's rows
+    // of the output against the golden's, through the library's own accuracy gate
+    int verdict = 0;
+    {
+        std::vector<float> gold((size_t)rows * n);
+        FILE *f = std::fopen((dir + "/golden.bin").c_str(), "rb");
+        if (f != nullptr) {
+            const bool got = std::fseek(f, (long)((size_t)rankId * gold.size() * sizeof(float)), SEEK_SET) == 0 &&
+                             std::fread(gold.data(), sizeof(float), gold.size(), f) == gold.size();
+            std::fclose(f);
+            if (got) {
+                std::vector<float> outF(out.size());
+                for (size_t i = 0; i < out.size(); ++i) {   // bf16 bit pattern -> fp32
+                    const uint32_t u = (uint32_t)out[i] << 16;
+                    std::memcpy(&outF[i], &u, 4);
+                }
+                uint64_t nBad = 0;
+                double mean = 0.0;
+                const int pass = catcoc_verify(outF.data(), gold.data(), outF.size(), BF16, k, &nBad, &mean);
+                std::printf("[verify] rank %u: %s (%llu of %zu elements outside rtol, mean relative error %.3e)\n", rankId,
+                            pass ? "PASS" : "FAIL", (unsigned long long)nBad, outF.size(), mean);
+                verdict = pass ? 0 : 4;
+            }
+        }
+    }
+
     for (float *p : peers) (void)hipFree(p);
     (void)hipFree(x1); (void)hipFree(x2); (void)hipFree(s1); (void)hipFree(s2);
     if (bias) (void)hipFree(bias);
     (void)hipFree(cAccum); (void)hipFree(dOut);
     (void)hipStreamDestroy(stream);
-    return 0;
+    return verdict;
 }

@@ -158,6 +158,33 @@ CATCOC_HD void comm_block_idx(uint32_t dir, uint32_t P, uint32_t splitRow, uint3
     rankIdx = r;
 }
 
+// BlockCommSwizzle<dir, deterministic> (comm_block_swizzle.hpp:25-31,54-56,114-118,147-186).  The deterministic
+// variant folds the npu split into the data split (coreSplit = {row * col, 1}) and pads the last band to the full
+// band width, so that core c of `row * col` cores meets every data block c, c + cores, ... with the ranks in a fixed
+// sequence; data indices at or beyond dataLoopsInRank are padding (GetActualBlockShape returns an empty block there).
+CATCOC_HD uint32_t comm_core_loop(bool deterministic, uint32_t P, uint32_t splitRow, uint32_t splitCol, uint32_t dataLoopsInRank)
+{
+    if (!deterministic) return dataLoopsInRank * P;
+    const uint32_t cores = splitRow * splitCol;
+    return ceil_div(dataLoopsInRank, cores) * cores * P;
+}
+
+CATCOC_HD void comm_block_idx_ex(uint32_t dir, bool deterministic, uint32_t P, uint32_t splitRow, uint32_t splitCol,
+                                 uint32_t dataLoopsInRank, uint32_t task, uint32_t &dataIdx, uint32_t &rankIdx)
+{
+    if (!deterministic) {
+        comm_block_idx(dir, P, splitRow, splitCol, dataLoopsInRank, task, dataIdx, rankIdx);
+        return;
+    }
+    const uint32_t cores = splitRow * splitCol;                    // direction 0 only: bands of `cores` data blocks
+    const uint32_t padded = ceil_div(dataLoopsInRank, cores) * cores;
+    const uint32_t inner = task % (padded * P);
+    uint32_t d, r;
+    banded_walk(cores, padded, P, inner, false, d, r);
+    dataIdx = d;
+    rankIdx = (r + d) % P;                                         // nStride = P / 1: (r * P) % P + (r * P) / P = r
+}
+
 // ---------------------------------------------------------------------------
 // Task -> tile of each operator
 // ---------------------------------------------------------------------------

@@ -69,6 +69,8 @@ EXPORTS = [
     "catcoc_default_tiling", "catcoc_swizzle_block_coord", "catcoc_splitk_block_coord", "catcoc_splitk_actual_k", "catcoc_splitk_launch_task",
     "catcoc_allgather_block_coord", "catcoc_comm_block_idx", "catcoc_task_tile", "catcoc_workgroup_task", "catcoc_launch_task", "catcoc_launch_tile",
     "catcoc_device_info", "catcoc_version",
+    "catcoc_pipelined_quant_matmul_reduce_scatter", "catcoc_pipelined_matmul_reduce_scatter", "catcoc_reduce_add",
+    "catcoc_verify", "catcoc_comm_block_idx_ex", "catcoc_comm_core_loop",
 ]
 
 _lib = None
@@ -165,6 +167,18 @@ def load():
     L.catcoc_device_info.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_char_p, C.c_int]
     L.catcoc_device_info.restype = C.c_int
     L.catcoc_version.restype = C.c_char_p
+    L.catcoc_pipelined_quant_matmul_reduce_scatter.argtypes = [vp, vp, C.c_uint64] + [vp] * 8 + [C.POINTER(CocTilingParams), u32, u32, u32, u32]
+    L.catcoc_pipelined_quant_matmul_reduce_scatter.restype = None
+    L.catcoc_pipelined_matmul_reduce_scatter.argtypes = [vp, vp, C.c_int] + [vp] * 4 + [C.POINTER(CocTilingParams), u32, u32, u32]
+    L.catcoc_pipelined_matmul_reduce_scatter.restype = None
+    L.catcoc_reduce_add.argtypes = [vp, vp, vp, C.c_uint64, u32, u32]
+    L.catcoc_reduce_add.restype = None
+    L.catcoc_verify.argtypes = [vp, vp, C.c_uint64, C.c_int, u32, C.POINTER(C.c_uint64), C.POINTER(C.c_double)]
+    L.catcoc_verify.restype = C.c_int
+    L.catcoc_comm_block_idx_ex.argtypes = [u32] * 7 + [pu, pu]
+    L.catcoc_comm_block_idx_ex.restype = None
+    L.catcoc_comm_core_loop.argtypes = [u32] * 5
+    L.catcoc_comm_core_loop.restype = u32
     _lib = L
     return L
 

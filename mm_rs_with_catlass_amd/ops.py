@@ -320,6 +320,109 @@ def allgather_matmul(a_local, peer_shards, b, rank=0, rank_size=1, tiling=None, 
                      workspace, split_k)
 
 
+def pipelined_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias, peers, rank, rank_size, outbound, c_accum=None,
+                                          out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0, deterministic=True,
+                                          comm_stream=None, block_num=0, stages=0, swizzle=None, out=None):
+    """The W8A8 operator in the reference's round-pipelined form (catcoc_pipelined_quant_matmul_reduce_scatter): GEMM rounds
+    on torch's current stream, comm rounds (int32 peers added into c_accum) and the dequant pass on comm_stream.
+    peers: rank_size-1 int32 partials [m/rank_size, n]; outbound: the symmetric workspace (bytes per
+    catcoc_get_workspace_size).  Returns (d_out, c_accum)."""
+    _check_rank(rank, rank_size)
+    _want(x1, "x1", torch.int8, 2)
+    _want(x2, "x2", torch.int8, 2)
+    m, k = x1.shape
+    n = x2.shape[0] if trans_b else x2.shape[1]
+    if (x2.shape[1] if trans_b else x2.shape[0]) != k:
+        _fail("x2 has shape %s: its k extent does not match x1's k = %d", tuple(x2.shape), k)
+    if m % rank_size != 0:
+        _fail("reduce-scatter needs m %% rank_size == 0 (m=%d, rank_size=%d)", m, rank_size)
+    rows = m // rank_size
+    _want(scale_x1, "scale_x1", torch.float32, 1, m)
+    _want(scale_x2, "scale_x2", torch.float32, 1, n)
+    _want(bias, "bias", torch.int32, 1, n)
+    _check_peers(list(peers), rank_size - 1, torch.int32, peer_row_offset + rows, n)
+    _want(outbound, "outbound", (torch.int32, torch.float32))
+    if c_accum is None:
+        c_accum = torch.empty((rows, n), dtype=torch.int32, device=x1.device)
+    _want(c_accum, "c_accum", torch.int32, 2, None, (rows, n))
+    if out is None:
+        out = torch.empty((rows, n), dtype=out_dtype, device=x1.device)
+    _want(out, "out", (torch.float16, torch.bfloat16), 2, None, (rows, n))
+    _check_dev(x1, x2, scale_x1, scale_x2, bias, outbound, c_accum, out, *peers)
+    t = tiling if tiling is not None else default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
+    d = _desc(rank, rank_size, list(peers), peer_row_offset, 0, block_num, stages, swizzle, outbound, None, None)
+    cs = comm_stream if comm_stream is not None else torch.cuda.current_stream()
+    _l.load().catcoc_pipelined_quant_matmul_reduce_scatter(
+        _stream(), cs.cuda_stream, 0, x1.data_ptr(), x2.data_ptr(), scale_x1.data_ptr(), scale_x2.data_ptr(), _ptr(bias),
+        c_accum.data_ptr(), out.data_ptr(), C.addressof(d), C.byref(t), 0, int(trans_b), _TORCH_TO_DT[out.dtype], int(deterministic))
+    _l.check()
+    return out, c_accum
+
+
+def pipelined_matmul_reduce_scatter(a, b, peers, rank, rank_size, outbound, tiling=None, trans_a=False, trans_b=False,
+                                    peer_row_offset=0, deterministic=True, comm_stream=None, block_num=0, stages=0, swizzle=None,
+                                    out=None, acc_dump=None):
+    """fp16 / bf16 reduce-scatter in the reference's round-pipelined form and precision: the local partial is rounded to the
+    16-bit type, peers are 16-bit partials [m/rank_size, n] of the same type, every add rounds to that type."""
+    if a.dtype not in _TORCH_TO_DT or b.dtype != a.dtype:
+        _fail("a and b must both be float16 or both bfloat16")
+    _check_rank(rank, rank_size)
+    _want(a, "a", None, 2)
+    _want(b, "b", None, 2)
+    m = a.shape[1] if trans_a else a.shape[0]
+    k = a.shape[0] if trans_a else a.shape[1]
+    n = b.shape[0] if trans_b else b.shape[1]
+    if (b.shape[1] if trans_b else b.shape[0]) != k:
+        _fail("b has shape %s: its k extent does not match a's k = %d", tuple(b.shape), k)
+    if m % rank_size != 0:
+        _fail("reduce-scatter needs m %% rank_size == 0 (m=%d, rank_size=%d)", m, rank_size)
+    rows = m // rank_size
+    _check_peers(list(peers), rank_size - 1, a.dtype, peer_row_offset + rows, n)
+    _want(outbound, "outbound", torch.float32)
+    if out is None:
+        out = torch.empty((rows, n), dtype=a.dtype, device=a.device)
+    _want(out, "out", a.dtype, 2, None, (rows, n))
+    _want(acc_dump, "acc_dump", torch.float32, None, m * n)
+    _check_dev(a, b, outbound, out, acc_dump, *peers)
+    t = tiling if tiling is not None else default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
+    d = _desc(rank, rank_size, list(peers), peer_row_offset, 0, block_num, stages, swizzle, outbound, None, acc_dump)
+    cs = comm_stream if comm_stream is not None else torch.cuda.current_stream()
+    _l.load().catcoc_pipelined_matmul_reduce_scatter(_stream(), cs.cuda_stream, _TORCH_TO_DT[a.dtype], a.data_ptr(), b.data_ptr(),
+                                                     out.data_ptr(), C.addressof(d), C.byref(t), int(trans_a), int(trans_b), int(deterministic))
+    _l.check()
+    return out
+
+
+def reduce_add(src, out_dtype=None, out=None):
+    """SplitkMatmul's ReduceAdd: src [slices, ...] fp32 -> sum over the slices in slice order, cast once to out_dtype
+    (None keeps fp32)."""
+    _want(src, "src", torch.float32)
+    if src.dim() < 2:
+        _fail("src must have the slices as its first dimension")
+    f, count = src.shape[0], src[0].numel()
+    dt = torch.float32 if out_dtype is None else out_dtype
+    if out is None:
+        out = torch.empty(src.shape[1:], dtype=dt, device=src.device)
+    _want(out, "out", dt, None, count)
+    _check_dev(src, out)
+    _l.load().catcoc_reduce_add(_stream(), out.data_ptr(), src.data_ptr(), count, f, 0 if dt == torch.float32 else _TORCH_TO_DT[dt])
+    _l.check()
+    return out
+
+
+def verify(out, gold, dtype, compute_times):
+    """The reference's accuracy gate on host data (float32 numpy arrays or CPU tensors).  -> (passed, n_bad, mean_rel_err)."""
+    import numpy as np
+    o = np.ascontiguousarray(out.numpy() if hasattr(out, "numpy") else out, dtype=np.float32).ravel()
+    g = np.ascontiguousarray(gold.numpy() if hasattr(gold, "numpy") else gold, dtype=np.float32).ravel()
+    if o.size != g.size:
+        _fail("out has %d elements, gold %d", o.size, g.size)
+    nb, eb = C.c_uint64(), C.c_double()
+    okv = _l.load().catcoc_verify(o.ctypes.data, g.ctypes.data, o.size, _TORCH_TO_DT.get(dtype, dtype), compute_times, C.byref(nb), C.byref(eb))
+    _l.check()
+    return bool(okv), nb.value, eb.value
+
+
 def kslice_plan(comm_type, dtype, m, k, n, rank=0, rank_size=1, tiling=None, split_k=0):
     """(workspace bytes, k slices) with which a launch of this shape would cut its tiles' k range; (0, 1) = it would not.
     m is the first dimension the operator's tiling takes (all-gather: one shard's rows)."""

@@ -57,7 +57,7 @@ def lib():
         _LIB.oracle_bf16_to_f32.argtypes = [C.c_uint16]
         _LIB.oracle_f16_to_f32.argtypes = [C.c_uint16]
         for name in ("oracle_splitk_first_ktile", "oracle_splitk_actual_k", "oracle_splitk_factor",
-                     "oracle_comm_block_row"):
+                     "oracle_comm_block_row", "oracle_comm_core_loop"):
             getattr(_LIB, name).restype = C.c_uint32
     return _LIB
 
@@ -258,6 +258,93 @@ def comm_block_idx(direction, P, splitRow, splitCol, dataLoopsInRank, task):
     lib().oracle_comm_block_idx(u32(direction), u32(P), u32(splitRow), u32(splitCol), u32(dataLoopsInRank),
                                 u32(task), C.byref(d), C.byref(r))
     return d.value, r.value
+
+
+def comm_core_loop(deterministic, P, splitRow, splitCol, dataLoopsInRank):
+    return lib().oracle_comm_core_loop(C.c_int(int(deterministic)), u32(P), u32(splitRow), u32(splitCol), u32(dataLoopsInRank))
+
+
+def comm_block_idx_det(P, splitRow, splitCol, dataLoopsInRank, task):
+    d, r = u32(), u32()
+    lib().oracle_comm_block_idx_det(u32(P), u32(splitRow), u32(splitCol), u32(dataLoopsInRank), u32(task), C.byref(d), C.byref(r))
+    return d.value, r.value
+
+
+def add_half(a_bits, b_bits, dtype):
+    a = _c(a_bits, np.uint16)
+    b = _c(b_bits, np.uint16)
+    out = np.empty(a.shape, np.uint16)
+    lib().oracle_add_half(_p(a), _p(b), C.c_size_t(a.size), C.c_int(dtype), _p(out))
+    return out
+
+
+def reduce_add(src_f32, dtype):
+    """src [slices, ...] fp32 -> the slices' sum in slice order, cast once (dtype 0: fp32)."""
+    src = _c(src_f32, np.float32)
+    f = src.shape[0]
+    count = src[0].size
+    out = np.empty(src.shape[1:], np.float32 if dtype == 0 else np.uint16)
+    lib().oracle_reduce_add(_p(src), C.c_size_t(count), u32(f), C.c_int(dtype), _p(out))
+    return out
+
+
+def pipelined_reduce_scatter_order(M, N, P, rank, m0, n0, blockNum, commInterval, commBlockM, splitRow, splitCol, off=7,
+                                   direction=1):
+    """The reference's comm rounds replayed on the CPU with the deterministic comm swizzle
+    (KQ:262-320 / KRS:237-296 with CSW's BlockCommSwizzle<0,true>): for every data block of every round, the rows and
+    columns of the kept block it covers and the ranks whose blocks are added to it, in the order its core meets them.
+    -> list of (row0, rows, col0, cols, [ranks])."""
+    mRank = M // P
+    loopsM, loopsN = -(-mRank // m0), -(-N // n0)
+    coreLoops = loopsM * loopsN * P
+    bpc = blockNum * commInterval
+    perRank = bpc // P
+    rounds = -(-coreLoops // bpc)
+    bpt = m0 // commBlockM
+    cores = splitRow * splitCol
+    blocks = []
+    for rnd in range(rounds):
+        actual = min(bpc, coreLoops - rnd * bpc)
+        dl = (actual // P) * bpt
+        loop = comm_core_loop(True, P, splitRow, splitCol, dl)
+        seq = {}
+        for core in range(cores):                      # a core runs its tasks one after the other (KQ:291)
+            for t in range(core, loop, cores):
+                d, r = comm_block_idx_det(P, splitRow, splitCol, dl, t)
+                if d >= dl or r == rank:               # padding block / this rank's own data (KQ:300)
+                    continue
+                seq.setdefault(d, []).append(r)
+        for d in range(dl):
+            tile, sub = divmod(d, bpt)
+            mi, ni = swizzle_block_coord(off, direction, loopsM, loopsN, rnd * perRank + tile)
+            row0 = mi * m0 + sub * commBlockM
+            rows = max(0, min(commBlockM, mRank - row0))
+            cols = min(n0, N - ni * n0)
+            blocks.append((row0, rows, ni * n0, cols, seq.get(d, [])))
+    return blocks
+
+
+def pipelined_reduce_half(local_f32, peers_bits, dtype, M, P, rank, m0, n0, blockNum, commInterval, commBlockM, splitRow,
+                          splitCol):
+    """Float reduce-scatter in the reference's precision: the local fp32 partial of the kept block [M/P, N] is rounded to
+    the 16-bit type, then each peer's 16-bit block is added with one rounding per add, ranks in the deterministic comm
+    order.  peers_bits[s] is the block of rank s (s < rank) or s + 1.  -> uint16 [M/P, N]."""
+    local = _c(local_f32, np.float32)
+    N = local.shape[1]
+    out = f32_to_half(local, dtype)
+    covered = np.zeros(local.shape, np.int32)
+    for row0, rows, col0, cols, ranks in pipelined_reduce_scatter_order(M, N, P, rank, m0, n0, blockNum, commInterval,
+                                                                        commBlockM, splitRow, splitCol):
+        if rows <= 0:
+            continue
+        sl = (slice(row0, row0 + rows), slice(col0, col0 + cols))
+        covered[sl] += 1
+        v = out[sl]
+        for r in ranks:
+            v = add_half(v, _c(peers_bits[r if r < rank else r - 1][sl], np.uint16), dtype)
+        out[sl] = v
+    assert (covered == 1).all(), "the comm blocks must tile the kept block exactly once"
+    return out
 
 
 def rs_task(M, N, P, m0, n0, blockNum, commInterval, stages, t, off=7, direction=1):

@@ -506,6 +506,52 @@ ORACLE_API void oracle_comm_block_idx(uint32_t dir, uint32_t P, uint32_t splitRo
     *dataIdx = d; *rankIdx = r;
 }
 
+/* CSW:25-31,54-56,106-118,147-186  BlockCommSwizzle<0, true>: the deterministic variant.  coreSplit becomes
+ * (row * col, 1), so swizzleOffset = row * col and nStride = P; GetCoreLoop pads dataLoopsInRank up to a multiple of
+ * the core count and the last band is NOT narrowed, so data indices >= dataLoopsInRank occur (empty blocks). */
+ORACLE_API uint32_t oracle_comm_core_loop(int deterministic, uint32_t P, uint32_t splitRow, uint32_t splitCol,
+                                          uint32_t dataLoopsInRank)
+{
+    if (!deterministic) return dataLoopsInRank * P;
+    uint32_t cores = splitRow * splitCol;
+    return (dataLoopsInRank + cores - 1) / cores * cores * P;
+}
+
+ORACLE_API void oracle_comm_block_idx_det(uint32_t P, uint32_t splitRow, uint32_t splitCol, uint32_t dataLoopsInRank,
+                                          uint32_t task, uint32_t *dataIdx, uint32_t *rankIdx)
+{
+    uint32_t off = splitRow * splitCol;
+    uint32_t rankLoops = P, nStride = P / 1;
+    uint32_t inner = task % oracle_comm_core_loop(1, P, splitRow, splitCol, dataLoopsInRank);
+    uint32_t band = inner / (off * rankLoops);
+    uint32_t inBand = inner % (off * rankLoops);
+    uint32_t d = band * off + inBand % off;
+    uint32_t r = inBand / off;
+    r = (r * nStride) % rankLoops + (r * nStride) / rankLoops;
+    r = (r + d) % rankLoops;
+    *dataIdx = d; *rankIdx = r;
+}
+
+/* One 16-bit add as a hardware atomic add on fp16 / bf16 memory does it (KRS:261 under SetAtomicAdd<half>): the exact
+ * sum rounded once, to nearest even, to the 16-bit type.  Computed as the fp32 sum rounded to 16 bits: fp32 carries
+ * 24 significand bits, at least 2p + 2 for p = 11 (fp16) and p = 8 (bf16), so the double rounding is innocuous. */
+ORACLE_API void oracle_add_half(const uint16_t *a, const uint16_t *b, size_t n, int dtype, uint16_t *out)
+{
+    for (size_t i = 0; i < n; ++i) out[i] = f32_to_half(half_to_f32(a[i], dtype) + half_to_f32(b[i], dtype), dtype);
+}
+
+/* SPK:24-161  ReduceAdd: dst[i] = cast(((s0[i] + s1[i]) + s2[i]) + ...), slices `count` apart, fp32 adds, one RNE cast
+ * (dtype 0 keeps fp32 and writes 4-byte elements). */
+ORACLE_API void oracle_reduce_add(const float *src, size_t count, uint32_t slices, int dtype, void *dst)
+{
+    for (size_t i = 0; i < count; ++i) {
+        float s = src[i];
+        for (uint32_t k = 1; k < slices; ++k) s = s + src[(size_t)k * count + i];
+        if (dtype == 0) ((float *)dst)[i] = s;
+        else ((uint16_t *)dst)[i] = f32_to_half(s, dtype);
+    }
+}
+
 /* CSW:188-201 with layoutComm = Packed(1, dLoopsInRank, commBlockM) (KQ:257-258):
  * first row of a comm block inside one round's comm shape.  Scatter+Get and
  * Gather+Put address the slab of the CURRENT rank, the other two pairs the slab

@@ -424,3 +424,62 @@ def test_python_entry_points_reject_mistyped_or_short_operands():
         ops.allgather_matmul(a, [a.clone()], b, 0, 2, acc_dump=torch.zeros((M, N)))      # the gathered product has 2M rows
     with pytest.raises(L.CatcocError, match="must live on the GPU"):
         ops.matmul_reduce_scatter(a, b, peers, 0, P)
+
+
+def test_verify_gate_equals_oracle(so):
+    # catcoc_verify is host code of the product (the reference's verify_result.py runs on the host too); it must agree
+    # with the oracle's restatement on random data, on the tolerance edges and on NaN / Inf handling
+    from mm_rs_with_catlass_amd import ops
+    rng = np.random.default_rng(3)
+    for dtype, ct in ((L.FP16, 100), (L.FP16, 4096), (L.BF16, 100), (L.BF16, 4096)):
+        gold = (rng.standard_normal(5000) * 50).astype(np.float32)
+        for noise in (0.0, 1e-3, 5e-3, 2e-2):
+            out = (gold * (1 + noise * rng.standard_normal(5000))).astype(np.float32)
+            out[::97] = np.nan
+            gold2 = gold.copy()
+            gold2[5::131] = np.inf
+            want = oracle.verify(out, gold2, dtype, ct)
+            got = ops.verify(out, gold2, dtype, ct)
+            assert got[0] == want[0] and got[1] == want[1] and abs(got[2] - want[2]) <= 1e-12, (dtype, ct, noise)
+    # exactly on the element-wise bound passes, one step beyond fails (rtol 2^-8 for fp16, computeTimes < 2048)
+    g = np.array([4.0, 0.5], np.float32)
+    assert ops.verify(g + np.array([4.0 / 256, 1.0 / 256], np.float32), g, L.FP16, 10)[1] == 0
+    over = np.array([np.nextafter(np.float32(4.0 + 4.0 / 256), np.float32(5)), 0.5], np.float32)
+    assert ops.verify(over, g, L.FP16, 10)[1] == 1
+    # a bias below the element-wise bound still fails the mean test (2^-10 for fp16)
+    g = np.full(1000, 2.0, np.float32)
+    ok_, bad, eb = ops.verify(g * (1 + 1.0 / 512), g, L.FP16, 10)
+    assert bad == 0 and not ok_ and eb > 2.0 ** -10
+    with pytest.raises(L.CatcocError):
+        ops.verify(g, g, 5, 10)
+
+
+def test_comm_swizzle_variants_equal_oracle(so):
+    d, r = u32(), u32()
+    for (P, sr, sc, dl) in [(8, 20, 1, 50), (8, 10, 2, 50), (4, 3, 1, 7), (8, 256, 1, 16), (2, 5, 2, 11)]:
+        assert so.catcoc_comm_core_loop(1, P, sr, sc, dl) == oracle.comm_core_loop(True, P, sr, sc, dl)
+        assert so.catcoc_comm_core_loop(0, P, sr, sc, dl) == dl * P
+        for t in range(oracle.comm_core_loop(True, P, sr, sc, dl) + 5):
+            so.catcoc_comm_block_idx_ex(0, 1, P, sr, sc, dl, t, C.byref(d), C.byref(r))
+            assert (d.value, r.value) == oracle.comm_block_idx_det(P, sr, sc, dl, t), (P, sr, sc, dl, t)
+        if P % sc == 0:
+            for t in range(dl * P):
+                so.catcoc_comm_block_idx_ex(0, 0, P, sr, sc, dl, t, C.byref(d), C.byref(r))
+                assert (d.value, r.value) == oracle.comm_block_idx(0, P, sr, sc, dl, t)
+
+
+def test_pipelined_entry_points_reject_bad_arguments(so):
+    t = L.CocTilingParams(m=1024, k=256, n=512, rankSize=8, commInterval=1, commBlockM=48)
+    d = L.make_desc(0, 8, [16] * 7, outbound=4096, outbound_bytes=1 << 40)
+    so.catcoc_pipelined_quant_matmul_reduce_scatter(None, None, 0, 16, 16, 16, 16, None, 16, 16, C.addressof(d), C.byref(t), 0, 0, L.BF16, 1)
+    assert so.catcoc_last_status() != 0 and "commBlockM" in L.last_error()
+    t.commBlockM = 64
+    so.catcoc_pipelined_quant_matmul_reduce_scatter(None, None, 0, 16, 16, 16, 16, None, None, 16, C.addressof(d), C.byref(t), 0, 0, L.BF16, 1)
+    assert so.catcoc_last_status() != 0 and "c_accum" in L.last_error()
+    d2 = L.make_desc(0, 8, [16] * 7)
+    so.catcoc_pipelined_matmul_reduce_scatter(None, None, L.FP16, 16, 16, 16, C.addressof(d2), C.byref(t), 0, 0, 1)
+    assert so.catcoc_last_status() != 0 and "outbound" in L.last_error()
+    so.catcoc_reduce_add(None, 16, 16, 10, 2, 0)
+    assert so.catcoc_last_status() != 0 and "multiple of 4" in L.last_error()
+    so.catcoc_reduce_add(None, 16, 16, 16, 0, 0)
+    assert so.catcoc_last_status() != 0

@@ -640,6 +640,175 @@ def test_float_transposed_operands_general_kernel():
         _check_float(host16(out), want, full, oracle.FP16, K)
 
 
+# ------------------------------------------------ round-pipelined, reference-faithful form
+def _outbound_for(comm, dt_code, t, rank, P, dtype):
+    import ctypes as C
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    need = L.load().catcoc_get_workspace_size(comm, dt_code, C.byref(t), C.byref(d))
+    L.check()
+    return torch.zeros(need // 4, dtype=dtype, device=DEV)
+
+
+@pytest.mark.parametrize("case", [(2048, 512, 256, 8, 3, 16, 1, 64, True), (2048, 512, 256, 8, 3, 16, 1, 64, False),
+                                  (4096, 1024, 320, 8, 7, 64, 2, 32, True), (1024, 768, 192, 4, 0, 20, 3, 128, False),
+                                  (800, 264, 208, 8, 5, 8, 1, 64, True)])
+def test_pipelined_quant_equals_fused_int32_reduce_and_oracle(case):
+    # GEMM rounds on one stream, comm rounds (BlockCommSwizzle task list, int32 adds into c_accum) and the dequant pass on
+    # another, stage reuse guarded by events.  int32 adds are exact in any order, so both comm schedules must equal the
+    # oracle and the fused kernel's int32-reduce mode bit for bit.
+    _need_gpu()
+    M, N, K, P, rank, block_num, ci, cb, det = case
+    rng = np.random.default_rng(900 + M + ci)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.integers(-1000, 1000, N, dtype=np.int32)
+    rows = M // P
+    peers = [rng.integers(-2 ** 24, 2 ** 24, (rows, N), dtype=np.int32) for _ in range(P - 1)]
+    acc_want, out_want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, b, rank * rows, rows, peers, oracle.BF16, reduce_int32=True)
+    t = ops.default_tiling(M, K, N, P, m0=128, n0=256, k0=256, commInterval=ci, commBlockM=cb, commDataSplit=20, commNpuSplit=1)
+    import ctypes as C
+    d = L.make_desc(rank, P, [16] * (P - 1), block_num=block_num)
+    need = L.load().catcoc_get_workspace_size(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, C.byref(t), C.byref(d))
+    ob = torch.zeros(need // 4, dtype=torch.int32, device=DEV)
+    side = torch.cuda.Stream()
+    dx = [dev(x1), dev(x2), dev(s1), dev(s2), dev(b)]
+    dp = [dev(p) for p in peers]
+    for it in range(2):
+        out, cacc = ops.pipelined_quant_matmul_reduce_scatter(*dx, dp, rank, P, ob, tiling=t, deterministic=det, comm_stream=side,
+                                                              block_num=block_num)
+        torch.cuda.synchronize()
+        kept = acc_want[rank * rows:(rank + 1) * rows] + sum(peers)
+        assert np.array_equal(cacc.cpu().numpy(), kept), "reduced int32 block differs"
+        assert np.array_equal(host16(out), out_want), "dequantised output differs from the oracle"
+    fused = ops.quant_matmul_reduce_scatter(*dx, dp, rank, P, tiling=t, reduce_int32=True, block_num=block_num)
+    torch.cuda.synchronize()
+    assert torch.equal(fused.view(torch.int16), out.view(torch.int16))
+    # the other ranks' int32 tiles sit in the workspace ring where the reference puts them (stage = round % 2)
+    so = L.load()
+    ntasks = so.catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+    obh = ob.cpu().numpy().reshape(-1, 256)
+    bpc = (block_num or 256) * ci
+    last_round = (ntasks - 1) // bpc
+    tr, row, col, ws = (C.c_uint32() for _ in range(4))
+    checked = 0
+    for task in range(ntasks):
+        so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row), C.byref(col), C.byref(ws))
+        rnd = task // bpc
+        if tr.value == rank or rnd + 2 <= last_round:        # kept tiles go to c_accum; older rounds were overwritten
+            continue
+        r0, c0 = row.value, col.value
+        rv, cv = min(128, (tr.value + 1) * rows - r0), min(256, N - c0)
+        assert np.array_equal(obh[ws.value:ws.value + rv, :cv], acc_want[r0:r0 + rv, c0:c0 + cv]), task
+        checked += 1
+    assert checked > 0
+
+
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+@pytest.mark.parametrize("case", [(2048, 512, 256, 8, 2, 16, 1, 64), (1024, 1024, 320, 4, 3, 0, 1, 32), (4096, 512, 128, 8, 6, 32, 2, 128)])
+def test_pipelined_float_reduces_in_half_precision_deterministically(dtype, case):
+    # the reference's float reduce: local partial rounded to the 16-bit type, 16-bit peers, one rounding per add
+    # (matmul_reduce_scatter.hpp:261).  With the deterministic comm swizzle the order of every block's adds is fixed,
+    # so the result equals the oracle's replay of the comm rounds bit for bit, launch after launch.
+    _need_gpu()
+    M, N, K, P, rank, block_num, ci, cb = case
+    rng = np.random.default_rng(950 + M)
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.05)
+    rows = M // P
+    peers = [oracle.f32_to_half(rng.standard_normal((rows, N)).astype(np.float32), dtype) for _ in range(P - 1)]
+    t = ops.default_tiling(M, K, N, P, m0=128, n0=256, k0=256, commInterval=ci, commBlockM=cb, commDataSplit=24, commNpuSplit=1)
+    import ctypes as C
+    d = L.make_desc(rank, P, [16] * (P - 1), block_num=block_num)
+    need = L.load().catcoc_get_workspace_size(L.MATMUL_REDUCE_SCATTER, dtype, C.byref(t), C.byref(d))
+    ob = torch.zeros(need // 4, dtype=torch.float32, device=DEV)
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    side = torch.cuda.Stream()
+    dA, dB, dP = dev16(A, dtype), dev16(B, dtype), [dev16(p, dtype) for p in peers]
+    outs = []
+    for it in range(3):
+        out = ops.pipelined_matmul_reduce_scatter(dA, dB, dP, rank, P, ob, tiling=t, deterministic=True, comm_stream=side,
+                                                  block_num=block_num, acc_dump=dump)
+        torch.cuda.synchronize()
+        outs.append(host16(out))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    local = dump.cpu().numpy()
+    part = oracle.gemm_half_f32(A, B, dtype)
+    assert np.abs(local - part).max() <= 1e-2 * max(1.0, np.abs(part).max())         # the GEMM itself, fp32 accumulate
+    want = oracle.pipelined_reduce_half(local[rank * rows:(rank + 1) * rows], peers, dtype, M, P, rank, 128, 256, block_num or 256, ci, cb, 24, 1)
+    assert np.array_equal(outs[0], want), "half-precision reduce differs from the replay of the comm rounds"
+    # against the unrounded sum: the textbook bound of recursive summation with unit roundoff u of the 16-bit type,
+    # |error| <= P * u * (|local| + sum |peers|) (P roundings; the reference's own element-wise gate, two ulps of the
+    # result, is tighter than what reducing in half precision can promise when partials cancel), and no bias
+    pf = [oracle.half_to_f32(p, dtype) for p in peers]
+    full = part[rank * rows:(rank + 1) * rows] + sum(pf)
+    mag = np.abs(part[rank * rows:(rank + 1) * rows]) + sum(np.abs(x) for x in pf)
+    u = 2.0 ** -11 if dtype == oracle.FP16 else 2.0 ** -8
+    err = np.abs(oracle.half_to_f32(outs[0], dtype) - full)
+    assert (err <= 1.01 * P * u * mag + 1e-6).all()
+    _, _, eb = oracle.verify(oracle.half_to_f32(outs[0], dtype), full, dtype, K)
+    assert eb <= 2.0 ** -12, eb
+
+
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+def test_pipelined_float_atomic_schedule_on_exactly_summable_data(dtype):
+    # BlockCommSwizzle<0,false> with hardware 16-bit atomic adds, arrival order: checked where every partial sum is exactly
+    # representable (small integers), so any order gives the same bits
+    _need_gpu()
+    M, N, K, P, rank = 2048, 512, 64, 8, 4
+    rng = np.random.default_rng(77)
+    A = oracle.f32_to_half(rng.integers(-1, 2, (M, K)).astype(np.float32), dtype)
+    B = oracle.f32_to_half(rng.integers(-1, 2, (K, N)).astype(np.float32), dtype)
+    rows = M // P
+    peers = [oracle.f32_to_half(rng.integers(-8, 9, (rows, N)).astype(np.float32), dtype) for _ in range(P - 1)]
+    t = ops.default_tiling(M, K, N, P, m0=128, n0=256, k0=256, commInterval=1, commBlockM=64, commDataSplit=16, commNpuSplit=2)
+    import ctypes as C
+    d = L.make_desc(rank, P, [16] * (P - 1), block_num=16)
+    need = L.load().catcoc_get_workspace_size(L.MATMUL_REDUCE_SCATTER, dtype, C.byref(t), C.byref(d))
+    ob = torch.zeros(need // 4, dtype=torch.float32, device=DEV)
+    out = ops.pipelined_matmul_reduce_scatter(dev16(A, dtype), dev16(B, dtype), [dev16(p, dtype) for p in peers], rank, P, ob, tiling=t,
+                                              deterministic=False, comm_stream=torch.cuda.Stream(), block_num=16)
+    torch.cuda.synchronize()
+    part = oracle.half_to_f32(A, dtype)[rank * rows:(rank + 1) * rows] @ oracle.half_to_f32(B, dtype)
+    want = part + sum(oracle.half_to_f32(p, dtype) for p in peers)
+    assert np.abs(want).max() <= 256                                   # integers below 2^8: exact in bf16 and fp16
+    assert np.array_equal(oracle.half_to_f32(host16(out), dtype), want.astype(np.float32))
+
+
+@pytest.mark.parametrize("case", [(4, 1024 * 1024, None), (2, 4096 * 13, torch.float16), (7, 1000 * 4, torch.bfloat16), (1, 515, torch.bfloat16),
+                                  (3, 64, None)])
+def test_splitk_reduce_add_kernel(case):
+    # SplitkMatmul's ReduceAdd as a kernel of its own: slices summed in slice order in fp32, one cast
+    _need_gpu()
+    f, count, dt = case
+    rng = np.random.default_rng(f * 31 + count % 97)
+    src = (rng.standard_normal((f, count)) * 10).astype(np.float32)
+    got = ops.reduce_add(dev(src), dt)
+    torch.cuda.synchronize()
+    code = 0 if dt is None else (oracle.FP16 if dt == torch.float16 else oracle.BF16)
+    want = oracle.reduce_add(src, code)
+    if dt is None:
+        assert np.array_equal(got.cpu().numpy(), want)
+    else:
+        assert np.array_equal(host16(got), want)
+
+
+def test_cpp_host_written_against_the_kernel_template_facade():
+    # include/catcoc_hip/dgemm.hpp: the reference's Catcoc::DGemm::Kernel::* class templates with their Params, forwarding
+    # to the C ABI; the host program compares each operator bit for bit with the direct C-ABI launch
+    _need_gpu()
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(L.LIB_PATH)), "catcoc_facade_host")
+    assert os.path.exists(exe), "catcoc_facade_host is not built"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    for name in ("QuantMatmulReduceScatter", "MatmulReduceScatter fp16", "MatmulAllReduce fp16", "AllGatherMatmul fp16",
+                 "MatmulReduceScatter bf16", "MatmulAllReduce bf16", "AllGatherMatmul bf16"):
+        assert "PASS " + name in r.stdout, r.stdout
+    assert "facade ok" in r.stdout
+
+
 # ------------------------------------------------------------ full benchmark size
 def test_quant_config4_full_size_properties():
     """W8A8 benchmark config (M=8192, K=1792, N=4096, P=8) at full size.  The oracle checks a row sample

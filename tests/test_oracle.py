@@ -522,3 +522,96 @@ def test_verify_elementwise_rule_matches_reference_compare_data():
     for ct in (100, 4096):
         want = REF_G.ref_compare_data(_p(out), _p(gold), C.c_uint64(out.size), u32(ct))
         assert oracle.verify(out, gold, oracle.FP16, ct)[1] == want
+
+
+# ------------------------------------------- deterministic comm swizzle, 16-bit adds, split-K reduce-add
+def test_comm_swizzle_deterministic_hand_cases():
+    # comm_block_swizzle.hpp:25-31,54-56,106-118,147-186 with IS_DETERMINISTIC worked by hand for the quant example's
+    # split (20 x 1 cores), P = 8, 50 data blocks per rank: the band width is the core count (20), the last band is
+    # padded to it (60 blocks -> 480 tasks), nStride = P, so task t of band b is (data b*20 + t%20, rank (t/20 + data) % 8).
+    assert oracle.comm_core_loop(True, 8, 20, 1, 50) == 480 and oracle.comm_core_loop(False, 8, 20, 1, 50) == 400
+    f = lambda t: oracle.comm_block_idx_det(8, 20, 1, 50, t)
+    assert f(0) == (0, 0) and f(1) == (1, 1) and f(19) == (19, 3)
+    assert f(20) == (0, 1) and f(21) == (1, 2)                       # same data blocks, next rank step
+    assert f(160) == (20, 4) and f(170) == (30, 6)                   # band 1
+    assert f(320 + 15) == (55, 7) and f(320 + 20 + 15) == (55, 0)    # band 2: data 50..59 are padding (>= 50)
+    # the npu split folds into the data split: (10 x 2) behaves exactly like (20 x 1)
+    assert all(oracle.comm_block_idx_det(8, 10, 2, 50, t) == f(t) for t in range(480))
+    # what makes it deterministic: core c (tasks c, c + cores, ...) owns data blocks c, c + 20, ... and meets the ranks of a
+    # block in the fixed sequence (data + i) % P
+    for c in (0, 7, 19):
+        tasks = [f(t) for t in range(c, 480, 20)]
+        for band in range(3):
+            seq = tasks[band * 8:(band + 1) * 8]
+            d = band * 20 + c
+            assert seq == [(d, (d + i) % 8) for i in range(8)]
+    pairs = {f(t) for t in range(480)}
+    assert len(pairs) == 480 and {p for p in pairs if p[0] < 50} == {(d, r) for d in range(50) for r in range(8)}
+
+
+def test_add_half_is_the_correctly_rounded_sum():
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 1 << 16, 200000).astype(np.uint16)
+    b = rng.integers(0, 1 << 16, 200000).astype(np.uint16)
+    fin = np.isfinite(a.view(np.float16)) & np.isfinite(b.view(np.float16))
+    a, b = a[fin], b[fin]
+    with np.errstate(over="ignore"):
+        want = (a.view(np.float16) + b.view(np.float16))            # numpy float16 addition is IEEE round-to-nearest-even
+    got = oracle.add_half(a, b, oracle.FP16).view(np.float16)
+    ok = np.isfinite(want)
+    assert np.array_equal(got[ok].view(np.uint16), want[ok].view(np.uint16))
+    # bf16 against exact rational arithmetic: the sum of two bf16 values, rounded once to 8 significand bits
+    from fractions import Fraction
+    a = rng.integers(0, 1 << 16, 3000).astype(np.uint16)
+    b = rng.integers(0, 1 << 16, 3000).astype(np.uint16)
+    fa, fb = oracle.half_to_f32(a, oracle.BF16), oracle.half_to_f32(b, oracle.BF16)
+    got = oracle.half_to_f32(oracle.add_half(a, b, oracle.BF16), oracle.BF16)
+    checked = 0
+    for x, y, g in zip(fa, fb, got):
+        if not (np.isfinite(x) and np.isfinite(y) and np.isfinite(g)) or abs(float(x) + float(y)) < 2.0 ** -120:
+            continue
+        s = Fraction(float(x)) + Fraction(float(y))
+        if s == 0:
+            assert g == 0
+            continue
+        e = 0                                                        # s = m * 2^e with 2^7 <= |m| < 2^8, m rounded to nearest even
+        mag = abs(s)
+        while mag >= 256:
+            mag /= 2; e += 1
+        while mag < 128:
+            mag *= 2; e -= 1
+        fl = mag.numerator // mag.denominator
+        rem = mag - fl
+        if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+            fl += 1
+        want = float(fl) * 2.0 ** e * (1 if s > 0 else -1)
+        assert float(g) == want, (x, y, g, want)
+        checked += 1
+    assert checked > 2000
+
+
+def test_reduce_add_is_slice_sequential_fp32_with_one_cast():
+    rng = np.random.default_rng(6)
+    src = (rng.standard_normal((5, 37, 11)) * 100).astype(np.float32)
+    want = src[0].copy()
+    for k in range(1, 5):
+        want = (want + src[k]).astype(np.float32)
+    assert np.array_equal(oracle.reduce_add(src, 0), want)
+    assert np.array_equal(oracle.reduce_add(src, oracle.FP16), want.astype(np.float16).view(np.uint16))
+    assert np.array_equal(oracle.reduce_add(src, oracle.BF16), oracle.f32_to_half(want, oracle.BF16))
+    # order matters in fp32: the oracle adds slice 0 first
+    tricky = np.array([[1.0e8], [1.0], [-1.0e8]], np.float32)
+    assert oracle.reduce_add(tricky, 0)[0] == np.float32(np.float32(np.float32(1.0e8) + np.float32(1.0)) + np.float32(-1.0e8))
+
+
+def test_pipelined_order_tiles_the_kept_block_and_skips_self():
+    # config-4-like geometry at small scale: every comm block covered exactly once, P - 1 ranks each, never this rank
+    M, N, P, rank = 2048, 1024, 8, 5
+    blocks = oracle.pipelined_reduce_scatter_order(M, N, P, rank, 128, 256, 16, 1, 64, 20, 1)
+    cover = np.zeros((M // P, N), np.int32)
+    for row0, rows, col0, cols, ranks in blocks:
+        cover[row0:row0 + rows, col0:col0 + cols] += 1
+        assert sorted(ranks) == [r for r in range(P) if r != rank]
+    assert (cover == 1).all()
+    # the rotation: different blocks start with different ranks
+    assert len({tuple(b[4]) for b in blocks}) > 1
