@@ -10,6 +10,7 @@ in HBM before the timed region.  Prints ONE JSON line.
     python bench.py --mode copy     # plain 256 MiB device copy: the known-size kernel the HBM counters are scaled by
     python bench.py --mode decode   # BASELINE config 5: skinny-M sweep, K = N = 8192, GB/s per M (HBM-bound)
     python bench.py --mode float    # BASELINE configs 3 (fp16 reduce-scatter), 2 (bf16 all-gather) and 1 (fp16 all-reduce)
+    python bench.py --mode sweep    # dynamic_tiling's sweep protocol on the MI355X-side knobs; writes the reference's result.csv
 """
 import argparse
 import json
@@ -189,12 +190,63 @@ def float_configs(args, torch, L, ops, dev):
         sys.exit(3)
 
 
+def tiling_sweep(args, torch, L, ops, dev):
+    """dynamic_tiling's sweep on the MI355X-side knobs (mm_rs_with_catlass_amd/tuning.py): config 4, config 3 and the three
+    shapes of the reference's examples/dynamic_tiling/scripts/test_shapes.csv (fp16, B stored [n,k]); writes result.csv."""
+    from mm_rs_with_catlass_amd import tuning
+    g = torch.Generator(device=dev).manual_seed(20250101)
+    P = 8
+    rows_all = []
+    # config 4: W8A8 reduce-scatter
+    M, K, N = 8192, 1792, 4096
+    x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=g)
+    x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g)
+    s1 = torch.empty(M, device=dev).uniform_(0.005, 0.02, generator=g)
+    s2 = torch.empty(N, device=dev).uniform_(0.001, 0.01, generator=g)
+    peers = [torch.randn((M // P, N), device=dev, generator=g) for _ in range(P - 1)]
+    out = torch.empty((M // P, N), dtype=torch.bfloat16, device=dev)
+    cs = torch.zeros(4096, dtype=torch.int64, device=dev)
+
+    def mk_quant(t, swz, linear):
+        return ops.prepare_quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, 0, P, tiling=t, swizzle=swz, linear_order=linear,
+                                                       checksum=cs, out=out)[0]
+    rows_all += tuning.sweep_shape("QuantMatmulReduceScatter", mk_quant, M, K, N, P, 0, 0, PEAK_INT8_TOPS)
+    del x1, x2, peers
+    # float reduce-scatter shapes: config 3 (row-major B) and the reference's own perf shapes (B as [n,k])
+    shapes = [(4096, 1792, 4096, 0, 0), (8192, 27392, 4096, 0, 1), (7936, 12544, 6656, 0, 1), (8144, 5120, 1696, 0, 1)]
+    for (M, K, N, ta, tb) in shapes:
+        A = torch.randn((M, K), device=dev, generator=g).half()
+        B = (torch.randn((N, K) if tb else (K, N), device=dev, generator=g) * 0.02).half()
+        peers = [torch.randn((M // P, N), device=dev, generator=g) for _ in range(P - 1)]
+        out = torch.empty((M // P, N), dtype=torch.float16, device=dev)
+        csf = torch.zeros(8192, dtype=torch.float64, device=dev)
+        full = (M // P) % 128 == 0 and N % 256 == 0
+
+        def mk_float(t, swz, linear, A=A, B=B, peers=peers, out=out, csf=csf, tb=tb):
+            return lambda: ops.matmul_reduce_scatter(A, B, peers, 0, P, tiling=t, trans_b=bool(tb), swizzle=swz, linear_order=linear,
+                                                     checksum=csf, out=out)
+        rows_all += tuning.sweep_shape("MatmulReduceScatter", mk_float, M, K, N, P, ta, tb, PEAK_F16_TFLOPS, full_tiles=full)
+        del A, B, peers
+    path = args.csv or os.path.join(ROOT, "gpurun_out", "result.csv")
+    os.makedirs(os.path.dirname(path), exist_ok=True)
+    tuning.write_result_csv(path, rows_all)
+    best = tuning.best_results(rows_all)
+    c4 = [b for b in best if b["Op"] == "QuantMatmulReduceScatter"][0]
+    print(json.dumps({
+        "metric": "tiling sweep, best Time(us) per shape (warm-up %d, %d timed launches, mean)" % (tuning.WARM_UP_TIMES, tuning.PERF_TEST_CYCLE_TIMES),
+        "value": c4["TOPS"], "unit": "TOPS", "n_gpus": 1, "steps": tuning.PERF_TEST_CYCLE_TIMES, "warmup": tuning.WARM_UP_TIMES,
+        "ms_per_step": c4["Time(us)"] / 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+        "data": "synthetic", "config": {"workload": "dynamic_tiling sweep over m0 / tile order / commInterval; value = best of config 4",
+                                        "candidates_timed": len(rows_all), "csv": os.path.relpath(path, ROOT)},
+        "best": best}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode", "float"], default="kept",
+    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode", "float", "sweep"], default="kept",
                     help="kept: non-kept tiles are folded into checksums (BASELINE's literal outputs); "
                          "outbound: they are also stored as fp32 to the symmetric workspace")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -204,6 +256,7 @@ def main():
     ap.add_argument("--sets", type=int, default=4, help="independent input sets the launches rotate over (1 = same buffers every launch)")
     ap.add_argument("--sustained", type=int, default=300, help="launches of the untimed sustained block (0 = skip)")
     ap.add_argument("--no-other-mode", action="store_true", help="skip the secondary run of the other store mode")
+    ap.add_argument("--csv", default="", help="--mode sweep: where result.csv goes (default gpurun_out/result.csv)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (peers are staged in the same GPU's HBM); --gpus %d is not "
@@ -239,6 +292,9 @@ def main():
         return
     if args.mode == "float":
         float_configs(args, torch, L, ops, dev)
+        return
+    if args.mode == "sweep":
+        tiling_sweep(args, torch, L, ops, dev)
         return
     M, K, N, P, rank = 8192, 1792, 4096, 8, args.rank
     rows = M // P

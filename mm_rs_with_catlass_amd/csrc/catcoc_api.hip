@@ -280,7 +280,15 @@ struct SplitkPlan {
     GemmArgs args;
     uint32_t f, tiles, rowBlocks;
     uint64_t workspaceBytes;   // partial tiles + counters (0 when f == 1)
+    bool large;                // many rows: the 128x256 direct-to-LDS kernel in row-mask mode runs instead of the split-K kernel
 };
+
+// Explicit kept rows with at least this many rows of A run the 128x256 direct-to-LDS kernel (k-sliced through the same
+// workspace) when the shape has full tiles and the kept rows are whole 32-row blocks.  Measured at K = N = 8192 with kept
+// rows = M / 8: M = 1024 129 against 159 us, M = 512 105 against 76 us (its 32 kept tiles add the peers after a main loop
+// twice as long as the split-K kernel's, which prefetches them), M = 256 92 against 46 us.  n0 = 256 (with m0 0 or 128) in
+// the tiling asks for the large tile explicitly, n0 = 128 for the split-K kernel.
+constexpr uint32_t kLargeTileRows = 1024;
 
 int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uint32_t transA, uint32_t transB, SplitkPlan &sp)
 {
@@ -292,8 +300,15 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
     if (transA || transB) return fail(E_SHAPE, "the explicit-kept-rows (split-K) path takes row-major A [m,k] and B [k,n] only");
     if (t->k % 64 != 0 || t->n % 128 != 0)
         return fail(E_SHAPE, "the explicit-kept-rows (split-K) path needs k %% 64 == 0 and n %% 128 == 0 (k=%u, n=%u)", t->k, t->n);
-    if ((t->m0 != 0 && t->m0 != 128) || (t->n0 != 0 && t->n0 != 128))
-        return fail(E_TILING, "the split-K path runs 128x128 tiles; leave m0/n0 zero or pass 128 (m0=%u, n0=%u)", t->m0, t->n0);
+    const bool canLarge = t->m % 128 == 0 && t->n % 256 == 0 && d->keptRowBegin % 32 == 0 && d->keptRows % 32 == 0;
+    const bool wantLarge = t->n0 == 256 && (t->m0 == 0 || t->m0 == 128);
+    if (wantLarge && !canLarge)
+        return fail(E_TILING, "128x256 tiles with explicit kept rows need m %% 128 == 0, n %% 256 == 0 and kept rows in whole 32-row blocks "
+                              "(m=%u, n=%u, kept [%u,+%u))", t->m, t->n, d->keptRowBegin, d->keptRows);
+    sp.large = wantLarge || (t->n0 == 0 && t->m0 == 0 && canLarge && t->m >= kLargeTileRows);
+    if (!sp.large && ((t->m0 != 0 && t->m0 != 128) || (t->n0 != 0 && t->n0 != 128)))
+        return fail(E_TILING, "explicit kept rows run 128x128 tiles (split-K kernel) or 128x256 tiles; leave m0/n0 zero or pass one of those "
+                              "(m0=%u, n0=%u)", t->m0, t->n0);
     if (d->keptRows == 0 || (uint64_t)d->keptRowBegin + d->keptRows > t->m)
         return fail(E_DESC, "kept rows [%u,+%u) outside [0,%u)", d->keptRowBegin, d->keptRows, t->m);
     if (d->flags & CATCOC_FLAG_REDUCE_INT32) return fail(E_DESC, "the split-K path reduces fp32 peers after the dequant only");
@@ -328,6 +343,26 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
     const uint32_t cores = d->blockNum ? d->blockNum : kDefaultBlockNum;
     const uint32_t kTiles = ceil_div(t->k, 256u);
     sp.tiles = ceil_div(t->m, 128u) * (t->n / 128u);
+    if (sp.large) {
+        // one grid of 128x256 tiles over all of A's rows (no rank structure), k slices as for any few-tile launch
+        const uint32_t stages = d->workspaceStages ? d->workspaceStages : kDefaultStages;
+        a.sched = make_sched(OP_ALLREDUCE, t->m, t->n, 1, 128, 256, cores, 1, stages, off, dir);
+        a.flags |= GF_ROW_MASK;
+        const uint32_t T = a.sched.coreLoops, nkAll = t->k / 64u;
+        uint32_t f = 1;
+        if (d->splitK != 0) {
+            if (d->splitK > 8u || d->splitK > nkAll) return fail(E_TILING, "splitK %u: at most %u k slices here", d->splitK, umin(8u, nkAll));
+            f = d->splitK;
+        } else {
+            while (f * 2u <= 8u && T * f * 2u <= 256u && nkAll / (f * 2u) >= 8u) f *= 2u;
+        }
+        if (f > 1 && T > kMaxCountedTiles) return fail(E_TILING, "k slices: %u tiles exceed the %u the workspace counts", T, kMaxCountedTiles);
+        sp.f = f;
+        a.splitK = f > 1 ? f : 0;
+        sp.rowBlocks = 4;
+        sp.workspaceBytes = f > 1 ? kCounterBlockBytes + (uint64_t)T * f * (128u * 256u * 4u) : 0;
+        return 0;
+    }
     uint32_t f = d->splitK ? d->splitK : splitk_factor(t->m, t->n, t->k, cores, 128, 128, 256);
     if (f > kTiles) f = kTiles;
     if (f == 0) f = 1;
@@ -371,6 +406,15 @@ void launch_quant_splitk(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_
     a.bias = (const int32_t *)bias;
     a.cAccum = (int32_t *)c_accum;
     a.outDtype = outDataType;
+    if (sp.large) {
+        bool aligned = (uintptr_t)scale_x2 % 16 == 0 && (uintptr_t)d_out % 16 == 0 && (!bias || (uintptr_t)bias % 16 == 0) && a.peerLd % 4 == 0;
+        for (uint32_t s = 0; s < a.nPeers && aligned; ++s) aligned = (uintptr_t)a.peers[s] % 16 == 0;
+        if (!aligned) { fail(E_SHAPE, "128x256 tiles with explicit kept rows need 16-byte aligned scales, bias, peers and output"); return; }
+        const int el = launch_gemm_dma_i8(a, stream);
+        if (el) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)el)); return; }
+        ok();
+        return;
+    }
     const int e = launch_gemm_splitk_i8(a, (int)sp.rowBlocks, sp.tiles * sp.f, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
     ok();

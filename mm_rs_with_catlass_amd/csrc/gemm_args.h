@@ -15,6 +15,9 @@ enum : uint32_t {
     GF_OUTBOUND_STORE = 1u << 0,  // non-kept tiles are stored to `outbound` (else folded into `checksum`)
     GF_REDUCE_INT32 = 1u << 1,    // W8A8: peers are int32 and are added before the dequant
     GF_LINEAR_ORDER = 1u << 2,    // workgroup i runs task i
+    GF_ROW_MASK = 1u << 3,        // kept rows [keptBegin, +keptRows) are whole 32-row blocks that need not line up with tiles: the
+                                  // epilogue works per 32-row block, and `checksum` takes the rows that are not kept per 128 x 128
+                                  // block, index (row / 128) * (N / 128) + col / 128
 };
 
 struct GemmArgs {

@@ -64,9 +64,13 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 //   WM 4 -> 256x256 tile, 8 waves (128 KiB LDS, one workgroup per CU): half the L2 -> LDS traffic per MAC.
 //   TB   -> B is given as [n][k] (k contiguous, the layout of a weight matrix stored output-major): its tiles are then
 //           staged and read exactly like A's, rows of 64 bytes of k, and need no transposing LDS reads.
-template <uint32_t DT, int WM, bool TB = false>
+//   RM   -> explicit kept rows (GF_ROW_MASK): the kept rows are whole 32-row blocks anywhere in the row range, so a tile can
+//           hold kept and not-kept blocks; every per-row step of the epilogue is then decided per 32-row block of a wave
+//           (wave-uniform branches, no per-lane selects).  A separate instantiation: the other launches pay nothing for it.
+template <uint32_t DT, int WM, bool TB = false, bool RM = false>
 __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
 {
+    static_assert(!RM || (DT == DT_I8 && WM == 2 && !TB), "row-mask mode exists for the W8A8 128-row kernel");
     static_assert(WM == 2 || WM == 4, "supported geometries");
     using Acc = typename AccOf<DT>::type;
     constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
@@ -531,7 +535,16 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const uint32_t col0 = wn * 128 + c32;       // + 32*nb
     const uint32_t gcol0 = ti.col + col0;
     const uint32_t row_base = wm * 32 * MB + h * 4;
-    const bool kept = ti.row >= args.keptBegin && ti.row < args.keptBegin + args.keptRows;
+    bool kept = ti.row >= args.keptBegin && ti.row < args.keptBegin + args.keptRows;
+    // RM: bit mb is set when 32-row block mb of this wave is kept (the unsigned compare also rejects blocks above keptBegin:
+    // the difference wraps); the tile counts as kept when any of its rows is
+    uint32_t keptMb = 0;
+    if constexpr (RM) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            if ((ti.row + wm * 32 * MB + mb * 32 - args.keptBegin) < args.keptRows) keptMb |= 1u << mb;
+        kept = ti.row < args.keptBegin + args.keptRows && ti.row + BM > args.keptBegin;
+    }
     // W8A8 accumulators are dequantised in place (the registers then hold fp32 bit patterns); element accesses go
     // through scalar temporaries
     auto getf = [&](int mb, int nb, int r) -> float {
@@ -598,22 +611,54 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         }
     }
 
+    if constexpr (RM) {
+        if (args.checksum != nullptr) {
+            // the accumulators of the 32-row blocks that are not kept, per 128 x 128 block (one wave column each)
+            long long si = 0;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                long long sb = 0;   // (summed for every block and dropped for kept ones: no control flow around the accumulators)
+#pragma unroll
+                for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sb += acc[mb][nb][r];
+                si += (kept && (keptMb & (1u << mb))) ? 0ll : sb;
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) si += __shfl_xor(si, o, 64);
+            long long *red = (long long *)smem;
+            __syncthreads();   // every wave has left the main loop's LDS reads behind
+            if (lane == 0) red[w] = si;
+            __syncthreads();
+            if (tid < 2) {
+                long long t = 0;
+#pragma unroll
+                for (int i = 0; i < WM; ++i) t += red[2 * i + tid];
+                ((long long *)args.checksum)[(size_t)(ti.row / 128u) * (args.N / 128u) + ti.col / 128u + tid] = t;
+            }
+        }
+    }
+
     if (kept) {
+        // (RM: a tile that starts above keptBegin makes this wrap; it is only added to rows of kept blocks, where the sum
+        // is the row's index in the kept range again)
         const uint32_t out_row0 = ti.row - args.keptBegin;
         if constexpr (DT == DT_I8) {
             if (args.cAccum != nullptr) {
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
+                for (int mb = 0; mb < MB; ++mb) {
+                    if (RM && !(keptMb & (1u << mb))) continue;   // (stores only)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
-                        int32_t *o = args.cAccum + (size_t)(out_row0 + lrow) * args.N + gcol0;
+                        int32_t *o = args.cAccum + (size_t)(uint32_t)(out_row0 + lrow) * args.N + gcol0;
 #pragma unroll
                         for (int nb = 0; nb < 4; ++nb) {
                             const int iv = acc[mb][nb][r];
                             o[32 * nb] = iv;
                         }
                     }
+                }
             }
             // dequantise in place: per-channel scale first, then per-token, each product rounded on its own
 #pragma unroll
@@ -630,16 +675,20 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         }
 
         // one fp32 partial of the tile, added from global memory 32 rows (64 loads per lane) at a time
-        auto add_partial = [&](const float *base, int64_t ld) {
+        // (RM: a block that is not kept adds the first 32 kept rows of the peer instead -- valid memory, and its sums are
+        // never stored; skipping it would put control flow around the accumulators, which costs far more than the loads)
+        auto add_partial = [&](const float *base, int64_t ld, const float *firstKept) {
             const float *src = base + (size_t)row_base * ld + gcol0;
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
+                const float *srcb = src + (size_t)(mb * 32) * ld;
+                if constexpr (RM) srcb = (keptMb & (1u << mb)) ? srcb : firstKept + (size_t)(h * 4) * ld + gcol0;
                 float pv[16][4];
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
 #pragma unroll
                     for (int nb = 0; nb < 4; ++nb)
-                        pv[r][nb] = __builtin_nontemporal_load(src + (size_t)(mb * 32 + (r >> 2) * 8 + (r & 3)) * ld + 32 * nb);
+                        pv[r][nb] = __builtin_nontemporal_load(srcb + (size_t)((r >> 2) * 8 + (r & 3)) * ld + 32 * nb);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
@@ -648,8 +697,10 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
-        for (uint32_t p = 0; p < args.nPeers; ++p)
-            add_partial((const float *)args.peers[p] + (size_t)(args.peerRowOffset + out_row0) * args.peerLd, args.peerLd);
+        for (uint32_t p = 0; p < args.nPeers; ++p) {
+            const float *peer = (const float *)args.peers[p] + args.peerRowOffset * args.peerLd;
+            add_partial(peer + (int64_t)(int32_t)out_row0 * args.peerLd, args.peerLd, peer);
+        }
 
         // 16-bit output.  A lane holds single columns 32 apart, so storing from registers would write 64-byte
         // pieces (half a cache line each, 128 store instructions per lane).  Instead every wave turns its 64 x 128
@@ -672,9 +723,10 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         };
         if (args.outDtype == DT_BF16) stage_all([](float f) { return f32_to_bf16_bits(f); });
         else stage_all([](float f) { return f32_to_f16_bits(f); });
-        unsigned char *dwave = (unsigned char *)args.d + ((size_t)(out_row0 + wm * 32 * MB) * args.ldd + ti.col + wn * 128) * 2;
+        unsigned char *dwave = (unsigned char *)args.d + (((int64_t)(int32_t)out_row0 + wm * 32 * MB) * args.ldd + ti.col + wn * 128) * 2;
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
+            if constexpr (RM) if (!(keptMb & (1u << (j >> 3)))) continue;   // rows 4j .. 4j+3 of the wave: 32-row block j / 8
             const uint32_t wrow = j * 4 + (lane >> 4), chunk = lane & 15;
             const v4i v = *(const v4i *)(st + wrow * 256 + ((chunk * 16) ^ (((wrow >> 2) & 1) << 7)));
             *(v4i *)(dwave + (size_t)wrow * args.ldd * 2 + chunk * 16) = v;
@@ -698,7 +750,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
                     for (int nb = 0; nb < 4; ++nb) __builtin_nontemporal_store(getf(mb, nb, r), ob + (size_t)lrow * sp.n0 + 32 * nb);
                 }
             }
-    } else if (args.checksum != nullptr) {
+    } else if (!RM && args.checksum != nullptr) {
         // int64 sum of the int32 accumulators (W8A8) or double sum of the fp32 ones
         using Sum = typename std::conditional<DT == DT_I8, long long, double>::type;
         Sum *red = (Sum *)smem;   // the pool is free again

@@ -17,6 +17,9 @@ int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
     else if (args.transB)   // B as [n][k]
         hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
                            (hipStream_t)stream, args);
+    else if (args.flags & GF_ROW_MASK)   // explicit kept rows in whole 32-row blocks
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
+                           (hipStream_t)stream, args);
     else   // one workgroup per tile, or per k slice of a tile
         hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
                            (hipStream_t)stream, args);

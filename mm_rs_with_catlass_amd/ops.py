@@ -177,9 +177,10 @@ def quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
     return out
 
 
-def splitk_plan(m, k, n, rank_size, kept_row_begin, kept_rows, split_k=0, block_num=0):
-    """(workspace bytes, split factor, 128x128 tiles) of the skinny-M split-K path for this problem."""
-    t = default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
+def splitk_plan(m, k, n, rank_size, kept_row_begin, kept_rows, split_k=0, block_num=0, n0=0):
+    """(workspace bytes, k slices, 128x128 blocks) of the explicit-kept-rows path for this problem.  n0 = 128 asks for the
+    128x128 split-K kernel, 256 for the 128x256 kernel, 0 lets the library choose by the number of rows."""
+    t = default_tiling(m, k, n, rank_size, m0=128 if n0 else 0, n0=n0, k0=0)
     d = _l.make_desc(0, rank_size, block_num=block_num)
     d.keptRowBegin, d.keptRows, d.splitK = kept_row_begin, kept_rows, split_k
     f, tiles = C.c_uint32(), C.c_uint32()
@@ -190,7 +191,7 @@ def splitk_plan(m, k, n, rank_size, kept_row_begin, kept_rows, split_k=0, block_
 
 def prepare_quant_matmul_splitk(x1, x2, scale_x1, scale_x2, bias=None, peers=(), rank_size=1, kept_row_begin=0,
                                 kept_rows=None, out_dtype=torch.bfloat16, split_k=0, workspace=None, checksum=None,
-                                acc_dump=None, c_accum=None, peer_row_offset=0, block_num=0, swizzle=None, out=None):
+                                acc_dump=None, c_accum=None, peer_row_offset=0, block_num=0, swizzle=None, out=None, n0=0):
     """Skinny-M (decode) form of the W8A8 operator: x1 [m,k] with any m, the rank keeps rows
     [kept_row_begin, +kept_rows); peers are rank_size-1 fp32 partials [kept_rows, n].  Returns (launch, out)."""
     _check_rank(0, rank_size)
@@ -214,7 +215,7 @@ def prepare_quant_matmul_splitk(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
     _want(checksum, "checksum", torch.int64, None, -(-m // 128) * -(-n // 128))
     _want(out, "out", (torch.float16, torch.bfloat16), 2, None, (kr, n))
     _check_dev(x1, x2, scale_x1, scale_x2, bias, checksum, acc_dump, c_accum, workspace, out, *peers)
-    t = default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
+    t = default_tiling(m, k, n, rank_size, m0=128 if n0 else 0, n0=n0, k0=0)
     d = _desc(0, rank_size, list(peers), peer_row_offset, 0, block_num, 0, swizzle, None, checksum, acc_dump)
     d.keptRowBegin = kept_row_begin
     d.keptRows = kept_rows if kept_rows is not None else m

@@ -263,8 +263,16 @@ def test_workspace_size_queries(so):
     need, f, tiles = ops.splitk_plan(16, 8192, 8192, 8, 0, 2)
     assert (f, tiles) == (oracle.splitk_factor(16, 8192, 8192, 256, 128, 128, 256), 64)
     assert need == f * tiles * 128 * 128 * 4 + 65536    # counter block of a fixed size first, then the partial tiles
-    need, f, tiles = ops.splitk_plan(512, 8192, 8192, 8, 0, 64)
-    assert (need, f, tiles) == (0, 1, 256)
+    assert ops.splitk_plan(512, 8192, 8192, 8, 0, 64) == (0, 1, 256)                # the 128x128 split-K kernel below 1024 rows
+    need, f, tiles = ops.splitk_plan(512, 8192, 8192, 8, 0, 64, n0=256)  # on request: 128 tiles of 128x256, two k slices each
+    assert (need, f, tiles) == (65536 + 128 * 2 * 131072, 2, 256)
+    assert ops.splitk_plan(1024, 8192, 8192, 8, 0, 128) == (0, 1, 512)              # many rows: 256 tiles of 128x256, no slices
+    assert ops.splitk_plan(1024, 8192, 8192, 8, 0, 128, n0=128)[1:] == (1, 512)
+    assert ops.splitk_plan(128, 8192, 8192, 8, 0, 32, n0=256) == (65536 + 32 * 8 * 131072, 8, 64)
+    assert ops.splitk_plan(128, 8192, 8192, 8, 0, 16)[1:] == (oracle.splitk_factor(128, 8192, 8192, 256, 128, 128, 256), 64)
+    assert ops.splitk_plan(2048, 8192, 8192, 8, 8, 64)[1:] == (1, 1024)             # kept rows off the 32-row grid: split-K kernel
+    with pytest.raises(L.CatcocError, match="128x256 tiles with explicit kept rows"):
+        ops.splitk_plan(128, 8192, 8192, 8, 0, 16, n0=256)
     need, f, tiles = ops.splitk_plan(200, 1088, 256, 4, 100, 50, split_k=3)
     assert (f, tiles) == (3, 4) and need == 3 * 4 * 65536 + 65536
     with pytest.raises(L.CatcocError, match="kept rows"):
@@ -483,3 +491,26 @@ def test_pipelined_entry_points_reject_bad_arguments(so):
     assert so.catcoc_last_status() != 0 and "multiple of 4" in L.last_error()
     so.catcoc_reduce_add(None, 16, 16, 16, 0, 0)
     assert so.catcoc_last_status() != 0
+
+
+def test_sweep_csv_has_the_reference_columns_and_best_pick(tmp_path):
+    # examples/dynamic_tiling/include/tiling.h:114 header, get_best_res.py:73-83 best row = min Time(us) per (Op, M, K, N)
+    import csv
+    from mm_rs_with_catlass_amd import tuning
+    rows = []
+    for i, us in enumerate((90.0, 71.5, 80.0)):
+        rows.append({"Op": "QuantMatmulReduceScatter", "M": 8192, "K": 1792, "N": 4096, "Transpose A": 0, "Transpose B": 0, "commInterval": 1 + i,
+                     "commTileM": 64, "commBlockM": 64, "commNpuSplit": 1, "commDataSplit": 2, "Time(us)": us, "m0": 128, "swizzleOffset": 7,
+                     "swizzleDirection": 1, "linearOrder": 0, "kSlices": 1, "TOPS": 1.0, "peakFraction": 0.1})
+    rows.append(dict(rows[0], Op="MatmulReduceScatter", **{"Time(us)": 5.0}))
+    path = tmp_path / "result.csv"
+    tuning.write_result_csv(str(path), rows)
+    with open(path) as f:
+        header = f.readline().strip().split(",")
+        assert header[:12] == ["Op", "M", "K", "N", "Transpose A", "Transpose B", "commInterval", "commTileM", "commBlockM", "commNpuSplit",
+                               "commDataSplit", "Time(us)"]
+        assert len(list(csv.reader(f))) == 4
+    best = tuning.best_results(rows)
+    assert len(best) == 2 and {b["Time(us)"] for b in best} == {71.5, 5.0}
+    assert (tuning.WARM_UP_TIMES, tuning.PERF_TEST_CYCLE_TIMES) == (10, 3)      # examples/dynamic_tiling/include/info.h:22-23
+    assert (256, (7, 1), False, 1) in tuning.candidates(1024, True) and all(c[0] != 256 for c in tuning.candidates(1018, False))

@@ -284,7 +284,10 @@ def test_k_slice_rejections():
 @pytest.mark.parametrize("case", [(1, 512, 1024, 8, 0, 1, 0), (16, 512, 2048, 8, 0, 2, 0), (16, 384, 1024, 8, 6, 10, 4),
                                   (64, 256, 4096, 8, 8, 8, 0), (128, 640, 2048, 8, 112, 16, 0), (200, 256, 1088, 4, 100, 50, 3),
                                   (33, 128, 64, 2, 0, 33, 0), (512, 1024, 1024, 8, 0, 64, 2), (64, 256, 2048, 4, 0, 16, 8),
-                                  (48, 384, 1536, 1, 0, 48, 6), (256, 256, 320, 2, 128, 128, 0)])
+                                  (48, 384, 1536, 1, 0, 48, 6), (256, 256, 320, 2, 128, 128, 0),
+                                  # many rows with kept rows in whole 32-row blocks: 128x256 tiles, epilogue per 32-row block
+                                  (512, 512, 512, 4, 96, 160, 0), (384, 768, 1024, 8, 352, 32, 4), (512, 1024, 2048, 8, 448, 64, 0),
+                                  (512, 512, 512, 4, 100, 160, 0)])    # the same off the 32-row grid: split-K kernel
 def test_quant_skinny_m_splitk(case):
     # decode shapes: any m, explicit kept rows, k slices meet through the workspace; int32 sums are exact
     _need_gpu()
@@ -303,9 +306,13 @@ def test_quant_skinny_m_splitk(case):
     acc_dump = torch.full((M, N), -7, dtype=torch.int32, device=DEV)
     c_accum = torch.full((kr, N), -7, dtype=torch.int32, device=DEV)
     checksum = torch.zeros(tiles, dtype=torch.int64, device=DEV)
+    n0 = 256 if (M % 128 == 0 and N % 256 == 0 and kb % 32 == 0 and kr % 32 == 0 and M >= 256) else 0   # exercise the large-tile route
+    if n0:
+        need, fac, tiles = ops.splitk_plan(M, K, N, P, kb, kr, split_k=f, n0=n0)
+        ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=DEV)
     launch, out = ops.prepare_quant_matmul_splitk(dev(x1), dev(x2), dev(s1), dev(s2), dev(b), [dev(p) for p in peers], P,
                                                   kb, kr, split_k=f, workspace=ws, checksum=checksum, acc_dump=acc_dump,
-                                                  c_accum=c_accum)
+                                                  c_accum=c_accum, n0=n0)
     for it in range(2):                      # the second launch reuses the workspace the first one re-armed
         out.zero_()
         launch()
