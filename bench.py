@@ -210,7 +210,8 @@ def tiling_sweep(args, torch, L, ops, dev):
     def mk_quant(t, swz, linear):
         return ops.prepare_quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, 0, P, tiling=t, swizzle=swz, linear_order=linear,
                                                        checksum=cs, out=out)[0]
-    rows_all += tuning.sweep_shape("QuantMatmulReduceScatter", mk_quant, M, K, N, P, 0, 0, PEAK_INT8_TOPS)
+    progress = lambda msg: print(msg, file=sys.stderr, flush=True)
+    rows_all += tuning.sweep_shape("QuantMatmulReduceScatter", mk_quant, M, K, N, P, 0, 0, PEAK_INT8_TOPS, progress=progress)
     del x1, x2, peers
     # float reduce-scatter shapes: config 3 (row-major B) and the reference's own perf shapes (B as [n,k])
     shapes = [(4096, 1792, 4096, 0, 0), (8192, 27392, 4096, 0, 1), (7936, 12544, 6656, 0, 1), (8144, 5120, 1696, 0, 1)]
@@ -225,7 +226,7 @@ def tiling_sweep(args, torch, L, ops, dev):
         def mk_float(t, swz, linear, A=A, B=B, peers=peers, out=out, csf=csf, tb=tb):
             return lambda: ops.matmul_reduce_scatter(A, B, peers, 0, P, tiling=t, trans_b=bool(tb), swizzle=swz, linear_order=linear,
                                                      checksum=csf, out=out)
-        rows_all += tuning.sweep_shape("MatmulReduceScatter", mk_float, M, K, N, P, ta, tb, PEAK_F16_TFLOPS, full_tiles=full)
+        rows_all += tuning.sweep_shape("MatmulReduceScatter", mk_float, M, K, N, P, ta, tb, PEAK_F16_TFLOPS, full_tiles=full, progress=progress)
         del A, B, peers
     path = args.csv or os.path.join(ROOT, "gpurun_out", "result.csv")
     os.makedirs(os.path.dirname(path), exist_ok=True)

@@ -350,6 +350,11 @@ CATCOC_API uint32_t catcoc_comm_core_loop(uint32_t deterministic, uint32_t P, ui
 CATCOC_API int catcoc_task_tile(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
                                 uint32_t task, uint32_t *targetRank, uint32_t *row, uint32_t *col,
                                 uint32_t *wsRow);
+/* The same for tasks [firstTask, firstTask + count) in one call (the launch is planned once): fills the arrays that are not
+ * NULL and returns how many tasks of the range exist. */
+CATCOC_API uint32_t catcoc_task_tiles(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
+                                      uint32_t firstTask, uint32_t count, uint32_t *targetRank, uint32_t *row, uint32_t *col,
+                                      uint32_t *wsRow);
 /* The task workgroup `wg` of a launch runs: an XCD-aware order with the kept rank's tiles first (they are the
  * long ones).  A bijection on [0, task count);
  * 0xffffffff for wg out of range or rejected arguments.  No counterpart in the reference, where AI core i

@@ -827,6 +827,30 @@ int catcoc_task_tile(int commType, const CocTilingParams *tiling, const CatcocSy
     return 1;
 }
 
+uint32_t catcoc_task_tiles(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t firstTask, uint32_t count,
+                           uint32_t *targetRank, uint32_t *row, uint32_t *col, uint32_t *wsRow)
+{
+    Plan p;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
+    d = *desc;
+    d.flags &= ~CATCOC_OUTBOUND_MASK;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    const int dataType = commType == QUANT_MATMUL_REDUCE_SCATTER ? INT8 : FP16;
+    if (make_plan(commType, dataType, tiling, &d, 0, 0, p)) return 0;   // planned once for the whole range
+    ok();
+    uint32_t n = 0;
+    for (; n < count; ++n) {
+        TileInfo ti;
+        if (!task_tile(p.args.sched, firstTask + n, ti)) break;
+        if (targetRank) targetRank[n] = ti.targetRank;
+        if (row) row[n] = ti.row;
+        if (col) col[n] = ti.col;
+        if (wsRow) wsRow[n] = ti.wsRow;
+    }
+    return n;
+}
+
 int catcoc_launch_tile(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc, uint32_t wg, uint32_t *task,
                        uint32_t *targetRank, uint32_t *row, uint32_t *col, uint32_t *wsRow)
 {

@@ -732,24 +732,42 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             *(v4i *)(dwave + (size_t)wrow * args.ldd * 2 + chunk * 16) = v;
         }
     } else if (args.flags & GF_OUTBOUND_STORE) {
-        float *ob = (float *)args.outbound + (size_t)ti.wsRow * sp.n0 + col0;
+        // fp32 tile of another rank, to the tile-linear workspace (rows wsRow .., n0 columns).  A lane holds single columns
+        // 32 apart, so storing from registers takes 128 four-byte stores per lane, and a wave can only have 63 memory
+        // operations outstanding: the tile would leave in three write round trips.  Instead every wave turns its block
+        // around in its private 16 KiB of LDS, 32 rows at a time (4-byte writes in accumulator layout, 16-byte reads along
+        // the rows), and leaves in 32 sixteen-byte streaming stores per lane that each cover two whole 512-byte row
+        // segments.  Rows with bit 2 set (the upper half-wave of a write) are shifted by 128 bytes to other banks.
+        static_assert(NW * 16384 <= POOL, "one 16 KiB staging area per wave");
+        unsigned char *st = smem + w * 16384;
+        __syncthreads();   // every wave has left the main loop's LDS reads behind
+        float *obw = (float *)args.outbound + ((size_t)ti.wsRow + wm * 32 * MB) * sp.n0 + wn * 128;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+        for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
-                if constexpr (DT == DT_I8) {
-                    const float sM = sMv[mb][r];
+                const uint32_t wrow = (r >> 2) * 8 + h * 4 + (r & 3);   // row inside the 32-row block
+                float sM = 1.f;
+                if constexpr (DT == DT_I8) sM = sMv[mb][r];
 #pragma unroll
-                    for (int nb = 0; nb < 4; ++nb) {
+                for (int nb = 0; nb < 4; ++nb) {
+                    float v;
+                    if constexpr (DT == DT_I8) {
                         const int iv = acc[mb][nb][r];
-                        __builtin_nontemporal_store(__fmul_rn(__fmul_rn((float)iv, sN[nb]), sM), ob + (size_t)lrow * sp.n0 + 32 * nb);
+                        v = __fmul_rn(__fmul_rn((float)iv, sN[nb]), sM);
+                    } else {
+                        v = getf(mb, nb, r);
                     }
-                } else {
-#pragma unroll
-                    for (int nb = 0; nb < 4; ++nb) __builtin_nontemporal_store(getf(mb, nb, r), ob + (size_t)lrow * sp.n0 + 32 * nb);
+                    *(float *)(st + wrow * 512 + (((nb * 32 + c32) * 4) ^ (h << 7))) = v;
                 }
             }
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const uint32_t wrow = j * 2 + (lane >> 5), chunk = lane & 31;
+                const v4f v = *(const v4f *)(st + wrow * 512 + ((chunk * 16) ^ (((wrow >> 2) & 1) << 7)));
+                __builtin_nontemporal_store(v, (v4f *)(obw + (size_t)(mb * 32 + wrow) * sp.n0 + chunk * 4));
+            }
+        }
     } else if (!RM && args.checksum != nullptr) {
         // int64 sum of the int32 accumulators (W8A8) or double sum of the fp32 ones
         using Sum = typename std::conditional<DT == DT_I8, long long, double>::type;

@@ -70,7 +70,7 @@ EXPORTS = [
     "catcoc_allgather_block_coord", "catcoc_comm_block_idx", "catcoc_task_tile", "catcoc_workgroup_task", "catcoc_launch_task", "catcoc_launch_tile",
     "catcoc_device_info", "catcoc_version",
     "catcoc_pipelined_quant_matmul_reduce_scatter", "catcoc_pipelined_matmul_reduce_scatter", "catcoc_reduce_add",
-    "catcoc_verify", "catcoc_comm_block_idx_ex", "catcoc_comm_core_loop",
+    "catcoc_verify", "catcoc_comm_block_idx_ex", "catcoc_comm_core_loop", "catcoc_task_tiles",
 ]
 
 _lib = None
@@ -179,6 +179,8 @@ def load():
     L.catcoc_comm_block_idx_ex.restype = None
     L.catcoc_comm_core_loop.argtypes = [u32] * 5
     L.catcoc_comm_core_loop.restype = u32
+    L.catcoc_task_tiles.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32, u32] + [pu] * 4
+    L.catcoc_task_tiles.restype = u32
     _lib = L
     return L
 

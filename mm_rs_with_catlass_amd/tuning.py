@@ -55,7 +55,7 @@ def time_launch(fn, warm_up=WARM_UP_TIMES, cycles=PERF_TEST_CYCLE_TIMES):
 
 
 def sweep_shape(op, make_launch, m, k, n, rank_size, trans_a, trans_b, peak_tops, full_tiles=True, warm_up=WARM_UP_TIMES,
-                cycles=PERF_TEST_CYCLE_TIMES):
+                cycles=PERF_TEST_CYCLE_TIMES, progress=None):
     """Time every candidate of one shape.  make_launch(tiling, swizzle, linear) -> callable enqueuing one launch, or raises
     CatcocError for a candidate the library rejects (skipped).  Returns result rows (dicts keyed by the CSV columns)."""
     rows = []
@@ -69,6 +69,9 @@ def sweep_shape(op, make_launch, m, k, n, rank_size, trans_a, trans_b, peak_tops
             continue
         us = time_launch(fn, warm_up, cycles)
         tops = 2.0 * m * n * k / us / 1e6
+        if progress is not None:
+            progress("[TEST] %s M=%d K=%d N=%d m0=%d swizzle=<%d,%d> linear=%d commInterval=%d: %.1f us" % (
+                op, m, k, n, m0, swz[0], swz[1], int(linear), ci, us))
         rows.append({"Op": op, "M": m, "K": k, "N": n, "Transpose A": int(trans_a), "Transpose B": int(trans_b),
                      "commInterval": t.commInterval, "commTileM": t.commTileM, "commBlockM": t.commBlockM,
                      "commNpuSplit": t.commNpuSplit, "commDataSplit": t.commDataSplit, "Time(us)": round(us, 2),

@@ -514,3 +514,18 @@ def test_sweep_csv_has_the_reference_columns_and_best_pick(tmp_path):
     assert len(best) == 2 and {b["Time(us)"] for b in best} == {71.5, 5.0}
     assert (tuning.WARM_UP_TIMES, tuning.PERF_TEST_CYCLE_TIMES) == (10, 3)      # examples/dynamic_tiling/include/info.h:22-23
     assert (256, (7, 1), False, 1) in tuning.candidates(1024, True) and all(c[0] != 256 for c in tuning.candidates(1018, False))
+
+
+def test_task_tiles_batch_query_equals_single_queries(so):
+    t = L.CocTilingParams(m=8192, k=1792, n=4096, m0=128, n0=256, k0=256, commInterval=10, rankSize=8)
+    d = L.make_desc(3, 8, [16] * 7, block_num=20)
+    n = so.catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+    arr = [(u32 * n)() for _ in range(4)]
+    got = so.catcoc_task_tiles(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), 0, n, *arr)
+    assert got == n == 1024
+    one = [u32() for _ in range(4)]
+    for task in (0, 1, 199, 200, 777, 1023):
+        assert so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, *[C.byref(x) for x in one])
+        assert tuple(a[task] for a in arr) == tuple(x.value for x in one)
+        assert tuple(a[task] for a in arr) == (lambda r: (r[0], r[3], r[4], r[5]))(oracle.rs_task(8192, 4096, 8, 128, 256, 20, 10, 2, task))
+    assert so.catcoc_task_tiles(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), 1000, 100, None, arr[1], None, None) == 24
