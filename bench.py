@@ -10,6 +10,7 @@ in HBM before the timed region.  Prints ONE JSON line.
     python bench.py --mode copy     # plain 256 MiB device copy: the known-size kernel the HBM counters are scaled by
     python bench.py --mode decode   # BASELINE config 5: skinny-M sweep, K = N = 8192, GB/s per M (HBM-bound)
     python bench.py --mode float    # BASELINE configs 3 (fp16 reduce-scatter), 2 (bf16 all-gather) and 1 (fp16 all-reduce)
+    python bench.py --mode ceiling  # what the int8 matrix pipes sustain on this box without any memory traffic (power-limited)
     python bench.py --mode sweep    # dynamic_tiling's sweep protocol on the MI355X-side knobs; writes the reference's result.csv
 """
 import argparse
@@ -242,12 +243,50 @@ def tiling_sweep(args, torch, L, ops, dev):
         "best": best}))
 
 
+def mfma_ceiling(args, torch, L, dev):
+    """What the matrix pipes sustain on this box for the benchmark's operand distribution: the 128x256 kernel's inner loop
+    without any global-memory traffic (catcoc_probe_mfma_int8), with and without its LDS fragment reads, on uniform random
+    int8 (the benchmark's data) and on constant bytes."""
+    so = L.load()
+    g = torch.Generator(device=dev).manual_seed(20250101)
+    patterns = {"uniform int8 [-127,127]": torch.randint(-127, 128, (73728,), dtype=torch.int8, device=dev, generator=g),
+                "constant 1": torch.ones(73728, dtype=torch.int8, device=dev)}
+    sink = torch.zeros(512 * 256, dtype=torch.int32, device=dev)
+    steps = args.ceiling_steps
+    ops_per_launch = 512.0 * 4 * steps * 16 * 65536
+    res = []
+    for name, pat in patterns.items():
+        for lds in (1, 0):
+            def fn():
+                rc = so.catcoc_probe_mfma_int8(torch.cuda.current_stream().cuda_stream, lds, steps, pat.data_ptr(), sink.data_ptr())
+                assert rc == 0
+            for _ in range(args.warmup):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(args.steps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            sec = e0.elapsed_time(e1) / 1e3 / args.steps
+            res.append({"data": name, "lds_fragment_reads": bool(lds), "ms_per_launch": round(sec * 1e3, 4),
+                        "TOPS": round(ops_per_launch / sec / 1e12, 1), "frac_of_peak": round(ops_per_launch / sec / 1e12 / PEAK_INT8_TOPS, 4)})
+    head = res[0]
+    print(json.dumps({
+        "metric": "int8 MFMA ceiling of the box: inner loop of the 128x256 kernel without global-memory traffic", "value": head["TOPS"],
+        "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_launch"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "512 workgroups x 4 waves x %d k steps x 16 mfma_i32_32x32x32_i8; value = uniform random int8 with LDS reads" % steps},
+        "ceiling": res}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode", "float", "sweep"], default="kept",
+    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode", "float", "sweep", "ceiling"], default="kept",
                     help="kept: non-kept tiles are folded into checksums (BASELINE's literal outputs); "
                          "outbound: they are also stored as fp32 to the symmetric workspace")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -257,6 +296,7 @@ def main():
     ap.add_argument("--sets", type=int, default=4, help="independent input sets the launches rotate over (1 = same buffers every launch)")
     ap.add_argument("--sustained", type=int, default=300, help="launches of the untimed sustained block (0 = skip)")
     ap.add_argument("--no-other-mode", action="store_true", help="skip the secondary run of the other store mode")
+    ap.add_argument("--ceiling-steps", type=int, default=20000, help="--mode ceiling: k steps per launch of the probe")
     ap.add_argument("--csv", default="", help="--mode sweep: where result.csv goes (default gpurun_out/result.csv)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -296,6 +336,9 @@ def main():
         return
     if args.mode == "sweep":
         tiling_sweep(args, torch, L, ops, dev)
+        return
+    if args.mode == "ceiling":
+        mfma_ceiling(args, torch, L, dev)
         return
     M, K, N, P, rank = 8192, 1792, 4096, 8, args.rank
     rows = M // P

@@ -370,6 +370,14 @@ CATCOC_API int catcoc_launch_tile(int commType, const CocTilingParams *tiling, c
  * CATCOC_FLAG_LINEAR_ORDER); a bijection on [0,tasks). */
 CATCOC_API uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags);
 
+/* Measurement helper (no counterpart in the reference): the 128x256 W8A8 kernel's inner loop without its global-memory
+ * side -- 512 workgroups of four waves, sixteen 32x32x32 int8 MFMAs per wave and step, with (ldsReads != 0) or without
+ * the LDS fragment reads that feed them -- on the 73728 bytes at `pattern` (device memory, 16-byte aligned), which every
+ * workgroup copies into its LDS first.  sink: 512 * 256 * 4 bytes of device memory.  Ops of a launch:
+ * 512 * 4 * steps * 16 * 65536.  It measures what the matrix pipes sustain for that data on the box at hand (they are
+ * power-limited); bench.py --mode ceiling reports it next to the operator's rate.  Returns 0 on success. */
+CATCOC_API int catcoc_probe_mfma_int8(void *stream, uint32_t ldsReads, uint32_t steps, const uint8_t *pattern, uint8_t *sink);
+
 /* Library / device information: fills cuCount, clockMHz of the current device; returns 0 on success. */
 CATCOC_API int catcoc_device_info(int *cuCount, int *clockMHz, char *name, int nameLen);
 CATCOC_API const char *catcoc_version(void);

@@ -71,6 +71,7 @@ EXPORTS = [
     "catcoc_device_info", "catcoc_version",
     "catcoc_pipelined_quant_matmul_reduce_scatter", "catcoc_pipelined_matmul_reduce_scatter", "catcoc_reduce_add",
     "catcoc_verify", "catcoc_comm_block_idx_ex", "catcoc_comm_core_loop", "catcoc_task_tiles",
+    "catcoc_probe_mfma_int8",
 ]
 
 _lib = None
@@ -181,6 +182,8 @@ def load():
     L.catcoc_comm_core_loop.restype = u32
     L.catcoc_task_tiles.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32, u32] + [pu] * 4
     L.catcoc_task_tiles.restype = u32
+    L.catcoc_probe_mfma_int8.argtypes = [vp, u32, u32, vp, vp]
+    L.catcoc_probe_mfma_int8.restype = C.c_int
     _lib = L
     return L
 
