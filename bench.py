@@ -429,6 +429,35 @@ def main():
                  "algorithmic_bytes": int(o_bytes), "hbm_frac": round(o_bytes / o_kern / 1e9 / PEAK_HBM_GBS, 4),
                  "kept_block_equals_main_mode": same}
 
+    # the reference's own structure (rounds of GEMM tasks and of comm blocks on two streams, int32 reduce before the dequant,
+    # quant_matmul_reduce_scatter.hpp:150-351), as a third figure: same shape, int32 peers, the outbound workspace as staging
+    pipelined = None
+    if not args.no_other_mode:
+        st = sets[0]
+        ipeers = [torch.randint(-2 ** 20, 2 ** 20, (rows, N), dtype=torch.int32, device=dev, generator=g) for _ in range(P - 1)]
+        c_acc = torch.empty((rows, N), dtype=torch.int32, device=dev)
+        p_out = torch.empty((rows, N), dtype=torch.bfloat16, device=dev)
+        comm = torch.cuda.Stream()
+        ptil = ops.default_tiling(M, K, N, P, m0=128, n0=256, k0=256)
+        p_ws = torch.empty(so.catcoc_get_workspace_size(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, C.byref(ptil), C.byref(desc0)) // 4,
+                           dtype=torch.int32, device=dev)
+
+        def pstep():
+            ops.pipelined_quant_matmul_reduce_scatter(st["x1"], st["x2"], st["s1"], st["s2"], None, ipeers, rank, P, p_ws,
+                                                      c_accum=c_acc, tiling=ptil, comm_stream=comm, out=p_out)
+        for _ in range(3):
+            pstep()
+        torch.cuda.synchronize()
+        n_p = 10
+        t0 = time.perf_counter()
+        for _ in range(n_p):
+            pstep()
+        torch.cuda.synchronize()   # (both streams: the call's last event joins the comm stream back into the current one)
+        p_s = (time.perf_counter() - t0) / n_p
+        pipelined = {"ms_per_step": round(p_s * 1e3, 5), "TOPS": round(2.0 * M * N * K / p_s / 1e12, 2), "commInterval": int(ptil.commInterval),
+                     "note": "catcoc_pipelined_quant_matmul_reduce_scatter: GEMM rounds and comm rounds on two streams, int32 "
+                             "peers reduced before the dequant; wall time per call over %d calls" % n_p}
+
     # bounded parity check of the timed configuration: a row sample of the kept block against the oracle
     import numpy as np
     import oracle
@@ -480,6 +509,8 @@ def main():
     }
     if other is not None:
         line[other_mode] = other
+    if pipelined is not None:
+        line["pipelined"] = pipelined
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(M, N, K, P, rank, args.cpu_repeats)
     print(json.dumps(line))

@@ -38,6 +38,12 @@
  *   maps, int32 peer reduce               and KAR:146-179 (several rounds, a
  *                                         reversed narrow band); numpy with
  *                                         distinct peers and a row offset.
+ *   deterministic BlockCommSwizzle,     : cases worked by hand from CSW:114-118,
+ *   comm core loop                        166-170 (rank of step d is (i + d) mod P),
+ *                                         every (rank, block) pair visited once.
+ *   half-precision add (one rounding    : numpy float16, exact rational sums
+ *   per add), ReduceAdd                   rounded once (fractions), numpy fp32
+ *                                         slice-sequential sums.
  *   peer reduce order                   : defined by this build (local partial
  *                                         first, then peers in ascending slot
  *                                         order); the reference reduces with
