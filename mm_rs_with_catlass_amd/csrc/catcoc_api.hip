@@ -131,7 +131,11 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     plan.dtype = dt;
     plan.blockNum = blockNum;
     // (B as [n,k] runs the 128-row direct-to-LDS kernel when its rows of k are 16-byte multiples)
-    plan.dma = fastShape && !plan.edge && (m0 == 256 || (m0 == 128 && (!transB || ((uint64_t)t->k * es) % 16 == 0))) && !transA &&
+    // Ragged rows / columns on 128-row tiles: the direct-to-LDS kernel moves the edge tiles inwards (GF_RAGGED).  It needs a whole
+    // tile to move into, k in whole 64-byte steps, and the moved tile's first column on the 16-byte grid of B, D and the peers.
+    const bool ragged = plan.edge && m0 == 128 && mRank >= m0 && t->n >= n0 && ((uint64_t)t->k * es) % 64 == 0 && t->n % 8 == 0 &&
+                        (transB || ((uint64_t)t->n * es) % 16 == 0);
+    plan.dma = fastShape && (!plan.edge || ragged) && (m0 == 256 || (m0 == 128 && (!transB || ((uint64_t)t->k * es) % 16 == 0))) && !transA &&
                (m0 == 128 || !transB) && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
 
     GemmArgs &a = plan.args;
@@ -154,6 +158,7 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
         a.flags |= GF_REDUCE_INT32;
     }
     if (d->flags & CATCOC_FLAG_LINEAR_ORDER) a.flags |= GF_LINEAR_ORDER;
+    if (plan.dma && plan.edge) a.flags |= GF_RAGGED;
 
     // kept rows
     if (op == OP_REDUCE_SCATTER) {
@@ -211,7 +216,7 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     // two slices (their sum does not depend on which arrives last).  desc.splitK overrides the choice.
     plan.kSlices = 1;
     plan.kSliceBytes = 0;
-    if (plan.dma && m0 == 128 && d->keptRows == 0) {
+    if (plan.dma && !plan.edge && m0 == 128 && d->keptRows == 0) {
         const uint32_t T = a.sched.coreLoops, nkAll = (uint32_t)((uint64_t)t->k * es / 64u);
         const uint32_t fmax = dt == DT_I8 ? 8u : 2u;
         uint32_t f = 1;
@@ -509,7 +514,8 @@ void launch_pipelined(bool quant, int dataType, void *computeStream, void *commS
         if (!check_ptr_align(p, a, b)) p.variant = 0;
     }
     g.nPeers = 0;
-    const bool dma = !quant && p.dma && p.variant != 0 && (uintptr_t)b % 16 == 0 && (g.ldb * 2) % 16 == 0 && (uintptr_t)d_out % 16 == 0;
+    const bool dma = !quant && p.dma && !p.edge && p.variant != 0 && (uintptr_t)b % 16 == 0 && (g.ldb * 2) % 16 == 0 && (uintptr_t)d_out % 16 == 0;
+    g.flags &= ~(uint32_t)GF_RAGGED;   // (ragged problems run the bounds-checked kernel here)
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles and 16-byte aligned row-major operands"); return; }
 
     CommArgs c;

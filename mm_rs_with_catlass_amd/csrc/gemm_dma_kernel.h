@@ -67,10 +67,16 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 //   RM   -> explicit kept rows (GF_ROW_MASK): the kept rows are whole 32-row blocks anywhere in the row range, so a tile can
 //           hold kept and not-kept blocks; every per-row step of the epilogue is then decided per 32-row block of a wave
 //           (wave-uniform branches, no per-lane selects).  A separate instantiation: the other launches pay nothing for it.
-template <uint32_t DT, int WM, bool TB = false, bool RM = false>
+//   RG   -> ragged problems (GF_RAGGED): a tile with fewer than m0 valid rows or n0 valid columns is computed as a whole tile
+//           moved up / left until it ends at the edge of its rank's row block / of the matrix.  Every load stays in bounds,
+//           the main loop is unchanged, and the rows and columns it shares with the neighbouring tile come out bit for bit as
+//           that tile computes them (same operands, same k order), so writing them twice is harmless; only what is counted
+//           per task (checksums) or laid out per task (workspace stores) has to leave the overlap out.
+template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false>
 __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
 {
     static_assert(!RM || (DT == DT_I8 && WM == 2 && !TB), "row-mask mode exists for the W8A8 128-row kernel");
+    static_assert(!RG || (WM == 2 && !RM), "ragged mode exists for the 128-row kernel");
     static_assert(WM == 2 || WM == 4, "supported geometries");
     using Acc = typename AccOf<DT>::type;
     constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
@@ -129,6 +135,14 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         TileInfo tg;   // (a separate object: filled in place, the tile of both routes ends up in memory instead of registers)
         task_tile(sp, task, tg);
         ti = tg;
+    }
+    uint32_t shiftM = 0, shiftN = 0;   // RG: rows / columns at the start of the tile that belong to the neighbouring tile
+    if constexpr (RG) {
+        shiftM = sp.m0 - ti.rowsValid;
+        shiftN = sp.n0 - ti.colsValid;
+        ti.row -= shiftM;
+        ti.rowInRank -= shiftM;
+        ti.col -= shiftN;
     }
     // The kept tiles are the longest chain of a reduce-scatter launch (main loop, then the peers' partials):
     // their waves get priority over the other workgroup on the CU so that the chain starts its streaming early.
@@ -741,7 +755,8 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         static_assert(NW * 16384 <= POOL, "one 16 KiB staging area per wave");
         unsigned char *st = smem + w * 16384;
         __syncthreads();   // every wave has left the main loop's LDS reads behind
-        float *obw = (float *)args.outbound + ((size_t)ti.wsRow + wm * 32 * MB) * sp.n0 + wn * 128;
+        // (RG: the tile's own rows and columns start at (shiftM, shiftN) and go to workspace position (0, 0))
+        float *obw = (float *)args.outbound + ((int64_t)ti.wsRow + wm * 32 * MB - (int64_t)shiftM) * sp.n0 + wn * 128 - (int64_t)shiftN;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
@@ -765,6 +780,8 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             for (int j = 0; j < 16; ++j) {
                 const uint32_t wrow = j * 2 + (lane >> 5), chunk = lane & 31;
                 const v4f v = *(const v4f *)(st + wrow * 512 + ((chunk * 16) ^ (((wrow >> 2) & 1) << 7)));
+                if constexpr (RG)
+                    if (wm * 32 * MB + mb * 32 + wrow < shiftM || wn * 128 + chunk * 4 < shiftN) continue;
                 __builtin_nontemporal_store(v, (v4f *)(obw + (size_t)(mb * 32 + wrow) * sp.n0 + chunk * 4));
             }
         }
@@ -774,10 +791,31 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         Sum *red = (Sum *)smem;   // the pool is free again
         Sum si = 0;
         bool summed = false;
+        if constexpr (RG) {
+            if ((shiftM | shiftN) != 0) {   // the tile's own part only
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const bool rowOwn = row_base + mb * 32 + (r >> 2) * 8 + (r & 3) >= shiftM;
+#pragma unroll
+                        for (int nb = 0; nb < 4; ++nb) {
+                            const bool own = rowOwn && col0 + 32 * nb >= shiftN;
+                            if constexpr (DT == DT_I8) {
+                                const int iv = acc[mb][nb][r];
+                                si += own ? iv : 0;
+                            } else {
+                                si += own ? (double)getf(mb, nb, r) : 0.0;
+                            }
+                        }
+                    }
+                summed = true;
+            }
+        }
         if constexpr (DT == DT_I8) {
             // |accumulator| <= 128 * 128 * k (int8 admits -128), so without a bias four of them add in 32 bits for
             // k < 32768 (4 * 2^14 * 32767 < 2^31): a third of the 64-bit additions
-            if (args.bias == nullptr && args.K < 32768u) {
+            if (!summed && args.bias == nullptr && args.K < 32768u) {
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll

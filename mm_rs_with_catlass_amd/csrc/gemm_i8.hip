@@ -14,6 +14,10 @@ int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
 {
     if (args.sched.m0 == 256)
         hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
+    else if ((args.flags & GF_RAGGED) && args.transB)   // ragged last tile row / column: edge tiles moved inwards
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, false, true>), dim3(launch_positions(args)), dim3(256), 0, (hipStream_t)stream, args);
+    else if (args.flags & GF_RAGGED)
+        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, false, true>), dim3(launch_positions(args)), dim3(256), 0, (hipStream_t)stream, args);
     else if (args.transB)   // B as [n][k]
         hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
                            (hipStream_t)stream, args);

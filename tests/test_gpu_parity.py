@@ -150,6 +150,42 @@ def test_quant_rs_ragged_edges(shape):
     quant_case(np.random.default_rng(4), M, N, K, 8, 6, bias=True)
 
 
+@pytest.mark.parametrize("case", [(8 * 296, 1344, 512, 8, 6, False), (8 * 296, 1280, 192, 8, 0, True), (4 * 1064, 1088, 128, 4, 3, False),
+                                  (2 * 1024, 2112, 256, 2, 1, True)])
+def test_quant_rs_ragged_problem_on_many_tiles(case):
+    # ragged rows and/or columns with 64 or more full tiles: two launches over one launch order, the direct-to-LDS
+    # kernel on the full tiles and the bounds-checked kernel on the ragged ones; every tile's accumulators, the kept
+    # block, the checksums and the outbound tiles must come out as from one launch
+    import ctypes as C
+    M, N, K, P, rank, outbound = case
+    stages = 0      # (every case is a single round of at most 256 tasks: no workspace stage is reused)
+    r = quant_case(np.random.default_rng(90 + rank), M, N, K, P, rank, bias=True, launches=2, outbound=outbound, stages=stages)
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+    d = L.make_desc(rank, P, [16] * (P - 1), stages=stages)
+    so = L.load()
+    tr, row, col, ws = (C.c_uint32() for _ in range(4))
+    rows = M // P
+    seen_ragged = seen_full = 0
+    deq = oracle.dequant(r["acc"], r["s2"], r["s1"]) if outbound else None
+    ob = r["outbound"].cpu().numpy().reshape(-1, 256) if outbound else None
+    cs = r["checksum"].cpu().numpy()
+    for task in range(r["ntasks"]):
+        so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row), C.byref(col), C.byref(ws))
+        rv = min(128, (tr.value + 1) * rows - row.value)
+        cv = min(256, N - col.value)
+        seen_ragged += rv < 128 or cv < 256
+        seen_full += rv == 128 and cv == 256
+        if tr.value == rank:
+            continue
+        blk = r["acc"][row.value:row.value + rv, col.value:col.value + cv]
+        if outbound:
+            want = deq[row.value:row.value + rv, col.value:col.value + cv]
+            assert np.array_equal(ob[ws.value:ws.value + rv, :cv].view(np.uint32), want.view(np.uint32)), task
+        else:
+            assert cs[task] == int(blk.astype(np.int64).sum()), task
+    assert seen_ragged > 0 and seen_full >= 64 and r["ntasks"] <= 256
+
+
 @pytest.mark.parametrize("shape", [(32, 129, 100), (24, 7, 3), (4 * 23, 45, 68), (4, 128, 512)])
 def test_quant_rs_general_shapes(shape):
     # K not a multiple of 16 or N not a multiple of 4: the general kernel (incl. the reference's own
@@ -474,6 +510,44 @@ def test_float_reduce_scatter(dtype, shape):
     _check_float(host16(out), want, full, dtype, K)
     pd = dump.cpu().numpy()
     assert np.abs(pd - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
+
+
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+def test_float_ragged_problems_on_many_tiles(dtype):
+    # full tiles on the direct-to-LDS kernel, ragged ones on the bounds-checked kernel, in two launches
+    _need_gpu()
+    rng = np.random.default_rng(26)
+    # reduce-scatter: 8 ranks x (2 full + 1 ragged) tile rows x (5 full + 1 ragged) tile columns
+    M, N, K, P, rank = 8 * 296, 1344, 224, 8, 5
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    part, want = oracle.matmul_reduce(A, B, dtype, rank * rows, rows, peers, want_partial=True)
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    out = ops.matmul_reduce_scatter(dev16(A, dtype), dev16(B, dtype), [dev(p) for p in peers], rank, P, acc_dump=dump)
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part[rank * rows:(rank + 1) * rows] + sum(peers), dtype, K)
+    assert np.abs(dump.cpu().numpy() - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
+    # all-gather with ragged shards and B as [n,k]
+    ml, N, K, P, rank = 424, 1024, 512, 8, 2
+    shards = [_rand16(rng, (ml, K), dtype) for _ in range(P)]
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    want = oracle.allgather_matmul(shards, B, dtype)
+    dsh = [dev16(s, dtype) for s in shards]
+    Bt = dev16(np.ascontiguousarray(B.T), dtype)
+    out = ops.allgather_matmul(dsh[rank], [dsh[r] for r in range(P) if r != rank], Bt, rank, P, trans_b=True)
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, oracle.gemm_half_f32(np.concatenate(shards, 0), B, dtype), dtype, K)
+    # all-reduce, ragged rows only
+    M, N, K = 1100, 2048, 320
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    p1 = rng.standard_normal((M, N)).astype(np.float32)
+    part, want = oracle.matmul_reduce(A, B, dtype, 0, M, [p1], want_partial=True)
+    out = ops.matmul_allreduce(dev16(A, dtype), dev16(B, dtype), [dev(p1)], 0, 2)
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part + p1, dtype, K)
 
 
 @pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
