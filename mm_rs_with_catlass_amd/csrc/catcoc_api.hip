@@ -125,7 +125,9 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
                         ((uint64_t)t->k * es) % 128 == 0 && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
     if (m0 == 0) m0 = (mRank <= 64) ? 64 : 128;
     const bool dmaShape = can256 && m0 == 256;
-    const bool fastShape = dmaShape || n0 == 256 && (m0 == 64 || m0 == 128) && !transA && t->k % che == 0 && t->n % 4 == 0;
+    // (A as [k,m] exists in the 128-row direct-to-LDS kernel only: rows of m in whole 16-byte pieces, a rank's block on that grid)
+    const bool taOk = !transA || (m0 == 128 && ((uint64_t)t->m * es) % 16 == 0 && ((uint64_t)mRank * es) % 16 == 0);
+    const bool fastShape = dmaShape || n0 == 256 && (m0 == 64 || m0 == 128) && taOk && t->k % che == 0 && t->n % 4 == 0;
     plan.variant = fastShape ? (int)(m0 / 64) : 0;   // 4 (m0 = 256) exists only as the direct-to-LDS kernel
     plan.edge = !(mRank % m0 == 0 && t->n % n0 == 0 && t->k % (64 / es) == 0);
     plan.dtype = dt;
@@ -135,8 +137,9 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     // tile to move into, k in whole 64-byte steps, and the moved tile's first column on the 16-byte grid of B, D and the peers.
     const bool ragged = plan.edge && m0 == 128 && mRank >= m0 && t->n >= n0 && ((uint64_t)t->k * es) % 64 == 0 && t->n % 8 == 0 &&
                         (transB || ((uint64_t)t->n * es) % 16 == 0);
-    plan.dma = fastShape && (!plan.edge || ragged) && (m0 == 256 || (m0 == 128 && (!transB || ((uint64_t)t->k * es) % 16 == 0))) && !transA &&
-               (m0 == 128 || !transB) && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
+    plan.dma = fastShape && (!plan.edge || ragged) && (m0 == 256 || (m0 == 128 && (!transB || ((uint64_t)t->k * es) % 16 == 0))) &&
+               (m0 == 128 || (!transA && !transB)) && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
+    if (transA && !plan.dma) plan.variant = 0;   // the other fast kernels take A as [m,k] only
 
     GemmArgs &a = plan.args;
     memset(&a, 0, sizeof(a));
@@ -274,6 +277,7 @@ void launch_float(int commType, int dataType, void *stream, uint8_t *a, uint8_t 
     const bool dma = p.dma && p.variant != 0 && (uintptr_t)b % 16 == 0 && (p.args.ldb * 2) % 16 == 0 && (uintptr_t)c % 16 == 0;
     if (!dma) p.args.splitK = 0;   // the other kernels run every tile whole
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles and 16-byte aligned row-major operands"); return; }
+    if (!dma && p.args.transA) p.variant = 0;
     const int e = dma ? (p.dtype == DT_F16 ? launch_gemm_dma_f16(p.args, stream) : launch_gemm_dma_bf16(p.args, stream))
                       : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
@@ -453,6 +457,7 @@ void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uin
     for (uint32_t s = 0; s < p.args.nPeers && dma; ++s) dma = (uintptr_t)p.args.peers[s] % 16 == 0;
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles, 16-byte aligned row-major operands and fp32 peers"); return; }
     if (!dma) p.args.splitK = 0;   // the other kernels run every tile whole
+    if (!dma && p.args.transA) p.variant = 0;
     const int e = dma ? launch_gemm_dma_i8(p.args, stream) : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
     ok();
@@ -517,6 +522,7 @@ void launch_pipelined(bool quant, int dataType, void *computeStream, void *commS
     const bool dma = !quant && p.dma && !p.edge && p.variant != 0 && (uintptr_t)b % 16 == 0 && (g.ldb * 2) % 16 == 0 && (uintptr_t)d_out % 16 == 0;
     g.flags &= ~(uint32_t)GF_RAGGED;   // (ragged problems run the bounds-checked kernel here)
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles and 16-byte aligned row-major operands"); return; }
+    if (!dma && g.transA) p.variant = 0;
 
     CommArgs c;
     memset(&c, 0, sizeof(c));

@@ -11,18 +11,10 @@ int launch_gemm_bf16(const GemmArgs &args, int variant, bool edge, void *stream)
 // Full-tile path with direct-to-LDS copies (row-major operands, see gemm_dma_kernel.h): m0 = 128 or 256.
 int launch_gemm_dma_bf16(const GemmArgs &args, void *stream)
 {
-    if (args.sched.m0 == 256)
+    if (args.sched.m0 == 256) {
         hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
-    else if ((args.flags & GF_RAGGED) && args.transB)   // ragged last tile row / column: edge tiles moved inwards
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 2, true, false, true>), dim3(launch_positions(args)), dim3(256), 0, (hipStream_t)stream, args);
-    else if (args.flags & GF_RAGGED)
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 2, false, false, true>), dim3(launch_positions(args)), dim3(256), 0, (hipStream_t)stream, args);
-    else if (args.transB)   // B as [n][k]
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 2, true>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
-                           (hipStream_t)stream, args);
-    else   // one workgroup per tile, or per k slice of a tile
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 2>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
-                           (hipStream_t)stream, args);
-    return (int)hipGetLastError();
+        return (int)hipGetLastError();
+    }
+    return launch_dma_128<DT_BF16>(args, (hipStream_t)stream);
 }
 }  // namespace catcoc

@@ -72,11 +72,15 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 //           the main loop is unchanged, and the rows and columns it shares with the neighbouring tile come out bit for bit as
 //           that tile computes them (same operands, same k order), so writing them twice is harmless; only what is counted
 //           per task (checksums) or laid out per task (workspace stores) has to leave the overlap out.
-template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false>
+//   TA   -> A is given as [k][m] (m contiguous): its tiles are then staged as rows of k, 128 bytes or 128 two-byte elements
+//           of m each, and read with the transposing LDS reads B uses (an MFMA's A operand wants k contiguous per lane for
+//           its row, exactly as its B operand does for its column).
+template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false>
 __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
 {
     static_assert(!RM || (DT == DT_I8 && WM == 2 && !TB), "row-mask mode exists for the W8A8 128-row kernel");
     static_assert(!RG || (WM == 2 && !RM), "ragged mode exists for the 128-row kernel");
+    static_assert(!TA || (WM == 2 && !RM), "transposed A exists for the 128-row kernel");
     static_assert(WM == 2 || WM == 4, "supported geometries");
     using Acc = typename AccOf<DT>::type;
     constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
@@ -152,7 +156,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const int64_t ldaB = args.lda * ES, ldbB = args.ldb * ES;  // row pitches in bytes
     const bool gather = sp.op == OP_ALLGATHER;
     const unsigned char *Ag = (const unsigned char *)args.a[gather ? ti.targetRank : 0] +
-                              (int64_t)(gather ? ti.rowInRank : ti.row) * ldaB;
+                              (TA ? (int64_t)(gather ? ti.rowInRank : ti.row) * ES : (int64_t)(gather ? ti.rowInRank : ti.row) * ldaB);
     const unsigned char *Bg = (const unsigned char *)args.b + (TB ? (size_t)ti.col * ldbB : (size_t)ti.col * ES);
     // k steps (64 bytes of K each) of this workgroup: all of them, or its slice
     const uint32_t nkAll = args.K * ES / 64;
@@ -160,7 +164,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     if (kSlices > 1) {   // (at most 16 slices of fewer than 2^24 steps: 32-bit products)
         const uint32_t kFirst = nkAll * slice / kSlices;
         nk = nkAll * (slice + 1u) / kSlices - kFirst;
-        Ag += (size_t)kFirst * 64;
+        Ag += TA ? (size_t)kFirst * (64 / ES) * ldaB : (size_t)kFirst * 64;
         Bg += TB ? (size_t)kFirst * 64 : (size_t)kFirst * (64 / ES) * ldbB;
     }
 
@@ -170,15 +174,28 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     const uint32_t ws = __builtin_amdgcn_readfirstlane((uint32_t)w);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(CATCOC_LDS unsigned char *)smem;
     // A (128-row tiles): copy j covers rows 16j..16j+15; lane -> row 16j + lane/4, LDS chunk slot lane&3 holds k chunk slot^swz
+    // A given as [k][m], 1-byte elements (64 k rows x 128 bytes): copy j covers k rows 8j..8j+7; lane -> row 8j + lane/8, slot
+    // lane&7 holds chunk slot ^ (((row>>1)&3)<<1).  2-byte elements (32 k rows x 256 bytes): copy j covers k rows 4j..4j+3;
+    // lane -> row 4j + lane/16, slot lane&15 holds chunk slot ^ ((row&3)<<2).
     const unsigned char *gA[A_DMA];
 #pragma unroll
-    for (int jj = 0; jj < A_DMA; ++jj)
-        gA[jj] = Ag + (size_t)(16 * (w + NW * jj) + (lane >> 2)) * ldaB + (((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+    for (int jj = 0; jj < A_DMA; ++jj) {
+        if constexpr (!TA) {
+            gA[jj] = Ag + (size_t)(16 * (w + NW * jj) + (lane >> 2)) * ldaB + (((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+        } else if constexpr (ES == 1) {
+            const int row = 8 * (w + NW * jj) + (lane >> 3);
+            gA[jj] = Ag + (size_t)row * ldaB + (((lane & 7) ^ (((row >> 1) & 3) << 1)) * 16);
+        } else {
+            const int row = 4 * (w + NW * jj) + (lane >> 4);
+            gA[jj] = Ag + (size_t)row * ldaB + (((lane & 15) ^ ((row & 3) << 2)) * 16);
+        }
+    }
+    const size_t aStep = TA ? (size_t)(64 / ES) * ldaB : (size_t)64;
     auto issue_a = [&](uint32_t ldsStage) {   // next k step of A into the stage at LDS byte offset ldsStage
 #pragma unroll
         for (int jj = 0; jj < A_DMA; ++jj) {
             dma16_at(gA[jj], lds0 + ldsStage + (ws + NW * jj) * 1024);
-            gA[jj] += 64;
+            gA[jj] += aStep;
         }
     };
     // B, 1-byte elements: copy j covers k rows 4j..4j+3; lane -> row 4j + lane/16, LDS slot lane&15 holds column
@@ -335,9 +352,40 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         auto offB = [&](uint32_t s3) { return 3 * A_STAGE + s3 * B_STAGE; };
         const uint32_t a_lds = (wm * 32 * MB + c32) * 64;
         const uint32_t a_sw = (c32 >> 2) & 3;
+        // A as [k][m]: the transposing reads of B, with this wave's 32-row blocks in place of 32-column blocks
+        uint32_t at_lds[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            if constexpr (ES == 1) {
+                const int trow = ti16 >> 1, thalf = ti16 & 1;
+                const int q = wm * 2 * MB + mb * 2 + tch;
+                at_lds[mb] = (16 * h + trow) * 128 + ((q ^ (((trow >> 1) & 3) << 1)) * 16) + thalf * 8;
+            } else {
+                const int trow = ti16 >> 2, tq = ti16 & 3;
+                const int q = wm * 4 * MB + mb * 4 + tch * 2 + (tq >> 1);
+                at_lds[mb] = (8 * h + trow) * 256 + ((q ^ (trow << 2)) * 16) + (tq & 1) * 8;
+            }
+        }
+        constexpr int AT_KK = (ES == 1) ? 32 * 128 : 16 * 256;   // bytes of a stage per 32-byte k slab
+        constexpr int AT_HALF = (ES == 1) ? 8 * 128 : 4 * 256;   // second transpose read of a fragment
         auto load_a = [&](v4i (&af)[MB], const unsigned char *sa, int kk) {
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) af[mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
+            for (int mb = 0; mb < MB; ++mb) {
+                if constexpr (!TA) {
+                    af[mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
+                } else {
+                    const unsigned char *p = sa + at_lds[mb] + kk * AT_KK;
+                    v2i t0, t1;
+                    if constexpr (ES == 1) {
+                        t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
+                        t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + AT_HALF));
+                    } else {
+                        t0 = __builtin_bit_cast(v2i, __builtin_amdgcn_ds_read_tr16_b64_v4i16((CATCOC_LDS v4s16 *)p));
+                        t1 = __builtin_bit_cast(v2i, __builtin_amdgcn_ds_read_tr16_b64_v4i16((CATCOC_LDS v4s16 *)(p + AT_HALF)));
+                    }
+                    af[mb] = v4i{t0.x, t0.y, t1.x, t1.y};
+                }
+            }
         };
         issue_a(offA(0));
         issue_b(offB(0));
@@ -850,6 +898,25 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         }
     }
 
+}
+
+// Launch of the 128-row geometry: one instantiation per operand layout (A as [m][k] or [k][m], B as [k][n] or [n][k]) and
+// for ragged problems; one workgroup per tile, or per k slice of a tile.
+template <uint32_t DT>
+inline int launch_dma_128(const GemmArgs &args, hipStream_t s)
+{
+    const dim3 grid(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), block(256);
+    switch ((args.transA ? 4 : 0) | (args.transB ? 2 : 0) | ((args.flags & GF_RAGGED) ? 1 : 0)) {
+        case 0: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false>), grid, block, 0, s, args); break;
+        case 1: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, true, false>), grid, block, 0, s, args); break;
+        case 2: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, false, false>), grid, block, 0, s, args); break;
+        case 3: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, true, false>), grid, block, 0, s, args); break;
+        case 4: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, true>), grid, block, 0, s, args); break;
+        case 5: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, true, true>), grid, block, 0, s, args); break;
+        case 6: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, false, true>), grid, block, 0, s, args); break;
+        default: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, true, true>), grid, block, 0, s, args); break;
+    }
+    return (int)hipGetLastError();
 }
 
 }  // namespace catcoc

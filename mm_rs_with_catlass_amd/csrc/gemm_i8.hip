@@ -12,21 +12,15 @@ int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream)
 // m0 = 128 (4 waves, two workgroups per CU) or m0 = 256 (8 waves).
 int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
 {
-    if (args.sched.m0 == 256)
+    if (args.sched.m0 == 256) {
         hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
-    else if ((args.flags & GF_RAGGED) && args.transB)   // ragged last tile row / column: edge tiles moved inwards
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, false, true>), dim3(launch_positions(args)), dim3(256), 0, (hipStream_t)stream, args);
-    else if (args.flags & GF_RAGGED)
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, false, true>), dim3(launch_positions(args)), dim3(256), 0, (hipStream_t)stream, args);
-    else if (args.transB)   // B as [n][k]
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
-                           (hipStream_t)stream, args);
-    else if (args.flags & GF_ROW_MASK)   // explicit kept rows in whole 32-row blocks
+        return (int)hipGetLastError();
+    }
+    if (args.flags & GF_ROW_MASK) {   // explicit kept rows in whole 32-row blocks
         hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
                            (hipStream_t)stream, args);
-    else   // one workgroup per tile, or per k slice of a tile
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2>), dim3(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), dim3(256), 0,
-                           (hipStream_t)stream, args);
-    return (int)hipGetLastError();
+        return (int)hipGetLastError();
+    }
+    return launch_dma_128<DT_I8>(args, (hipStream_t)stream);
 }
 }  // namespace catcoc

@@ -109,13 +109,13 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
                                         out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
                                         reduce_int32=False, outbound=None, checksum=None, acc_dump=None,
                                         c_accum=None, block_num=0, stages=0, swizzle=None, linear_order=False,
-                                        out=None, workspace=None, split_k=0):
+                                        out=None, workspace=None, split_k=0, trans_a=False):
     """Validate and bind the arguments once; returns (launch, out) where launch() enqueues one call of
     catcoc_launch_quant_matmul_reduce_scatter on torch's current stream (for launch-rate-sensitive loops)."""
     _check_rank(rank, rank_size)
     _want(x1, "x1", torch.int8, 2)
     _want(x2, "x2", torch.int8, 2)
-    m, k = x1.shape
+    m, k = (x1.shape[1], x1.shape[0]) if trans_a else x1.shape
     n = x2.shape[0] if trans_b else x2.shape[1]
     if (x2.shape[1] if trans_b else x2.shape[0]) != k:
         _fail("x2 has shape %s: its k extent does not match x1's k = %d", tuple(x2.shape), k)
@@ -148,7 +148,7 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
     keep = (x1, x2, scale_x1, scale_x2, bias, tuple(peers), outbound, checksum, acc_dump, c_accum, out, d, t, workspace)
     fn = L.catcoc_launch_quant_matmul_reduce_scatter
     argv = (0, x1.data_ptr(), x2.data_ptr(), scale_x1.data_ptr(), scale_x2.data_ptr(), _ptr(bias), _ptr(c_accum),
-            out.data_ptr(), C.addressof(d), C.byref(t), 0, int(trans_b), _TORCH_TO_DT[out.dtype])
+            out.data_ptr(), C.addressof(d), C.byref(t), int(trans_a), int(trans_b), _TORCH_TO_DT[out.dtype])
 
     def launch(_keep=keep):
         fn(_stream(), *argv)
@@ -160,10 +160,10 @@ def quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
                                 out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
                                 reduce_int32=False, outbound=None, checksum=None, acc_dump=None, c_accum=None,
                                 block_num=0, stages=0, swizzle=None, linear_order=False, out=None, workspace=None,
-                                split_k=0):
+                                split_k=0, trans_a=False):
     """W8A8 matmul -> reduce-scatter share of one rank.
 
-    x1 [m,k] int8, x2 [k,n] int8 ([n,k] with trans_b), scale_x1 [m] fp32 per token, scale_x2 [n] fp32 per
+    x1 [m,k] int8 ([k,m] with trans_a), x2 [k,n] int8 ([n,k] with trans_b), scale_x1 [m] fp32 per token, scale_x2 [n] fp32 per
     channel, bias [n] int32 or None.  peers: rank_size-1 staged partials for the kept rows (fp32, or int32
     with reduce_int32), added in list order after the local partial.  workspace: optional zero-initialised uint8
     tensor of kslice_plan() bytes with which a launch of few tiles cuts its k range into slices.
@@ -171,7 +171,8 @@ def quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
     """
     launch, out = prepare_quant_matmul_reduce_scatter(
         x1, x2, scale_x1, scale_x2, bias, peers, rank, rank_size, out_dtype, tiling, trans_b, peer_row_offset,
-        reduce_int32, outbound, checksum, acc_dump, c_accum, block_num, stages, swizzle, linear_order, out, workspace, split_k)
+        reduce_int32, outbound, checksum, acc_dump, c_accum, block_num, stages, swizzle, linear_order, out, workspace, split_k,
+        trans_a)
     launch()
     _l.check()
     return out

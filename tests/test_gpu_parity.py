@@ -47,7 +47,7 @@ def ulp_diff16(a_bits, b_bits):
 TORCH_DT = {oracle.FP16: torch.float16, oracle.BF16: torch.bfloat16}
 
 
-def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, trans_b=False, reduce_int32=False,
+def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, trans_b=False, trans_a=False, reduce_int32=False,
                full_peers=False, tiling=None, outbound=False, block_num=0, stages=0, swizzle=None, linear=False,
                launches=1, kslices=None):
     _need_gpu()
@@ -67,6 +67,7 @@ def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, tran
         x1, x2, s1, s2, b, rank * rows, rows, peers, out_dtype, peer_row0=prow0, reduce_int32=reduce_int32)
 
     x2d = dev(np.ascontiguousarray(x2.T)) if trans_b else dev(x2)
+    x1d = dev(np.ascontiguousarray(x1.T)) if trans_a else dev(x1)
     acc_dump = torch.full((M, N), -7, dtype=torch.int32, device=DEV)
     c_accum = torch.full((rows, N), -7, dtype=torch.int32, device=DEV)
     dpeers = [dev(p) for p in peers]
@@ -94,8 +95,8 @@ def quant_case(rng, M, N, K, P, rank, *, bias=False, out_dtype=oracle.BF16, tran
         kw["split_k"] = kslices[0]
     for it in range(launches):
         out = ops.quant_matmul_reduce_scatter(
-            dev(x1), x2d, dev(s1), dev(s2), dev(b) if bias else None, dpeers, rank, P, out_dtype=TORCH_DT[out_dtype],
-            tiling=tiling, trans_b=trans_b, peer_row_offset=prow0, reduce_int32=reduce_int32, acc_dump=acc_dump,
+            x1d, x2d, dev(s1), dev(s2), dev(b) if bias else None, dpeers, rank, P, out_dtype=TORCH_DT[out_dtype],
+            tiling=tiling, trans_b=trans_b, trans_a=trans_a, peer_row_offset=prow0, reduce_int32=reduce_int32, acc_dump=acc_dump,
             c_accum=c_accum, block_num=block_num, stages=stages, swizzle=swizzle, linear_order=linear, **kw)
         torch.cuda.synchronize()
         if it + 1 < launches:
@@ -700,6 +701,50 @@ def test_float_weights_stored_n_by_k(dtype):
                                trans_b=True, workspace=ws)
     torch.cuda.synchronize()
     _check_float(host16(out), want, oracle.gemm_half_f32(np.concatenate(shards, 0), B, dtype), dtype, K)
+
+
+@pytest.mark.parametrize("case", [(2048, 512, 320, 4, 1, False, None), (2048, 512, 320, 4, 2, True, None), (8 * 304, 1344, 192, 8, 5, False, None),
+                                  (8 * 304, 1344, 192, 8, 0, True, None), (1024, 1024, 2048, 4, 1, False, (0, 4)), (32, 129, 100, 4, 3, False, None)])
+def test_quant_rs_activations_stored_k_by_m(case):
+    # A given as [k,m]: full and ragged problems on the direct-to-LDS kernel (A staged as rows of k and read through the
+    # transposing LDS reads), with either layout of B, also cut into k slices; anything else on the general kernel
+    M, N, K, P, rank, tb, ks = case
+    r = quant_case(np.random.default_rng(60 + rank), M, N, K, P, rank, bias=True, trans_a=True, trans_b=tb, launches=2, kslices=ks)
+    if M >= 1024:
+        assert r["exact"] == r["total"]
+
+
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+def test_float_activations_stored_k_by_m(dtype):
+    _need_gpu()
+    rng = np.random.default_rng(27)
+    for (M, N, K, P, rank) in ((2048, 512, 224, 4, 3), (8 * 296, 1344, 96, 8, 6)):
+        A = _rand16(rng, (M, K), dtype)
+        B = _rand16(rng, (K, N), dtype, 0.02)
+        rows = M // P
+        peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+        part, want = oracle.matmul_reduce(A, B, dtype, rank * rows, rows, peers, want_partial=True)
+        full = part[rank * rows:(rank + 1) * rows] + sum(peers)
+        At = dev16(np.ascontiguousarray(A.T), dtype)
+        for tb in (0, 1):
+            b = dev16(np.ascontiguousarray(B.T) if tb else B, dtype)
+            dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+            out = ops.matmul_reduce_scatter(At, b, [dev(p) for p in peers], rank, P, trans_a=True, trans_b=bool(tb), acc_dump=dump)
+            torch.cuda.synchronize()
+            _check_float(host16(out), want, full, dtype, K)
+            assert np.abs(dump.cpu().numpy() - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
+    # all-reduce, cut into two k slices
+    M, N, K = 1024, 512, 1024
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    p1 = rng.standard_normal((M, N)).astype(np.float32)
+    part, want = oracle.matmul_reduce(A, B, dtype, 0, M, [p1], want_partial=True)
+    need, f = ops.kslice_plan(L.MATMUL_ALLREDUCE, TORCH_DT[dtype], M, K, N, 0, 2)
+    assert f == 2
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    out = ops.matmul_allreduce(dev16(np.ascontiguousarray(A.T), dtype), dev16(B, dtype), [dev(p1)], 0, 2, trans_a=True, workspace=ws)
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part + p1, dtype, K)
 
 
 def test_float_transposed_operands_general_kernel():
