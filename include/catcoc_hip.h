@@ -270,7 +270,8 @@ CATCOC_API uint64_t catcoc_get_workspace_size(int commType, int dataType, const 
 /* Launches with few 128x256 tiles (fewer than half the CUs' worth) can cut every tile's k range into k slices, one
  * workgroup each, that meet through `workspace` (partial tiles in 32-bit words + one counter per tile, zeroed once
  * by the caller, re-armed by every launch): returns the bytes needed and the slice count (1 and 0 bytes when the
- * launch would not be sliced: other tile shapes, transposed or ragged operands, enough tiles already).  The count
+ * launch would not be sliced: other tile shapes, ragged problems, enough tiles already; the operands' layouts do
+ * not matter).  The count
  * is 2, 4 or 8 for W8A8 (integer partials add exactly) and at most 2 for fp16/bf16 (a two-term fp32 sum does not
  * depend on which slice arrives last); desc->splitK, when non-zero, is taken as the caller's own count.  A launch
  * slices only when `workspace` is given.  Counterpart in the reference: SplitkMatmul's k split
