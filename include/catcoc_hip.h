@@ -358,7 +358,9 @@ CATCOC_API uint32_t catcoc_task_tiles(int commType, const CocTilingParams *tilin
                                       uint32_t *wsRow);
 /* The task workgroup `wg` of a launch runs: an XCD-aware order with the kept rank's tiles first (they are the
  * long ones).  A bijection on [0, task count);
- * 0xffffffff for wg out of range or rejected arguments.  No counterpart in the reference, where AI core i
+ * 0xffffffff for wg out of range or rejected arguments.  (A reduce-scatter launch of at most 512 tiles with short
+ * k runs every kept tile as two 64-row workgroups, placed first in the same order; this function still describes
+ * the order by tile.)  No counterpart in the reference, where AI core i
  * simply runs tasks i, i + BLOCK_NUM, ... (quant_matmul_reduce_scatter.hpp:166-170). */
 CATCOC_API uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
                                        uint32_t wg);

@@ -75,16 +75,26 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 //   TA   -> A is given as [k][m] (m contiguous): its tiles are then staged as rows of k, 128 bytes or 128 two-byte elements
 //           of m each, and read with the transposing LDS reads B uses (an MFMA's A operand wants k contiguous per lane for
 //           its row, exactly as its B operand does for its column).
-template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false>
-__global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
+// One LDS pool per workgroup, carved by constant offsets:
+//   128-row tile: three A stages (8 KiB each), then three B stages (16 KiB each)            = 72 KiB
+//   256-row tile: two A pair buffers (32 KiB each), then four B stages (16 KiB each)         = 128 KiB
+// (a 64-row tile of the four-wave geometry uses the first 60 KiB of the 72)
+template <int WM> struct DmaPool { static constexpr int BYTES = (WM == 4) ? (4 * 256 * 64 + 4 * 64 * 256) : 3 * (128 * 64 + 64 * 256); };
+
+// One tile (or one k slice of a tile) of the launch: position `pos` of the launch order, in the caller's LDS pool.
+// MB = 32-row blocks per wave (2; 1 = a 64-row tile, four-wave geometry only); subRow = first row of a 64-row tile inside
+// its 128-row tile of the schedule.
+template <uint32_t DT, int WM, bool TB, bool RM, bool RG, bool TA, int MB>
+__device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *smem, uint32_t pos, uint32_t slice, uint32_t kSlices,
+                                         uint32_t subRow)
 {
     static_assert(!RM || (DT == DT_I8 && WM == 2 && !TB), "row-mask mode exists for the W8A8 128-row kernel");
     static_assert(!RG || (WM == 2 && !RM), "ragged mode exists for the 128-row kernel");
     static_assert(!TA || (WM == 2 && !RM), "transposed A exists for the 128-row kernel");
     static_assert(WM == 2 || WM == 4, "supported geometries");
+    static_assert(MB == 2 || (MB == 1 && WM == 2 && !RM && !RG && !TA), "64-row tiles exist for the plain four-wave geometry");
     using Acc = typename AccOf<DT>::type;
     constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
-    constexpr int MB = 2;
     constexpr int NW = 2 * WM;          // waves
     constexpr int BM = 32 * MB * WM;
     constexpr int A_STAGE = BM * 64;
@@ -92,12 +102,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     constexpr int A_DMA = BM / 16 / NW;  // 1 KiB copies per wave per stage
     constexpr int B_DMA = 16 / NW;
     constexpr int STEP_DMA = A_DMA + B_DMA;
-
-    // One LDS pool, carved by constant offsets:
-    //   BM = 128: three A stages (8 KiB each), then three B stages (16 KiB each)            = 72 KiB
-    //   BM = 256: two A pair buffers (32 KiB each), then four B stages (16 KiB each)         = 128 KiB
-    constexpr int POOL = (BM == 256) ? (4 * A_STAGE + 4 * B_STAGE) : 3 * (A_STAGE + B_STAGE);
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[POOL];
+    constexpr int POOL = DmaPool<WM>::BYTES;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -115,20 +120,6 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
                  "s"(sp.dPerRank.d), "s"(sp.dPerRank.m), "s"(sp.dStages.d), "s"(sp.dStages.m), "s"(sp.dBpc.d), "s"(sp.dBpc.m),
                  "s"(args.keptRank), "s"(args.flags), "s"(args.K), "s"(args.N));
     const bool linear = (args.flags & GF_LINEAR_ORDER) != 0;
-    // A launch with few tiles can cut every tile's k range into kSlices pieces, one workgroup each (128-row tiles
-    // only): position `pos` of the launch order runs as kSlices workgroups that stay in the position's XCD column.
-    uint32_t pos = blockIdx.x + args.taskBase, slice = 0;   // (taskBase is zero for k-sliced launches)
-    const uint32_t kSlices = (WM == 2 && args.splitK > 1) ? args.splitK : 1u;
-    if (kSlices > 1) {
-        if ((sp.coreLoops & 7u) == 0) {
-            const uint32_t q = blockIdx.x >> 3;
-            slice = q % kSlices;
-            pos = (q / kSlices) * 8u + (blockIdx.x & 7u);
-        } else {
-            slice = blockIdx.x % kSlices;
-            pos = blockIdx.x / kSlices;
-        }
-    }
     if (pos >= sp.coreLoops) return;
     uint32_t task;
     TileInfo ti;
@@ -139,6 +130,10 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         TileInfo tg;   // (a separate object: filled in place, the tile of both routes ends up in memory instead of registers)
         task_tile(sp, task, tg);
         ti = tg;
+    }
+    if constexpr (MB == 1) {
+        ti.row += subRow;
+        ti.rowInRank += subRow;
     }
     uint32_t shiftM = 0, shiftN = 0;   // RG: rows / columns at the start of the tile that belong to the neighbouring tile
     if constexpr (RG) {
@@ -296,6 +291,37 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     CATCOC_FENCE();
     // read_a(af, kk): A fragments of this step; sb: B stage of this step; slot1/2/3/4: the step's other work
     auto sched_step = [&](auto read_a, const unsigned char *sb, auto slot1, auto slot2, auto slot3, auto slot4) {
+        if constexpr (MB == 1) {   // eight MFMAs per step: the same lag of half a step, two reads per gap
+            CATCOC_MMA(fa1, fb1, 0, 0)
+            read_a(fa0, 0);
+            read_b1(fb0, sb, 0, 0);
+            CATCOC_FENCE();
+            CATCOC_MMA(fa1, fb1, 0, 1)
+            read_b1(fb0, sb, 0, 1);
+            read_b1(fb0, sb, 0, 2);
+            CATCOC_FENCE();
+            CATCOC_MMA(fa1, fb1, 0, 2)
+            read_b1(fb0, sb, 0, 3);
+            slot1();
+            CATCOC_FENCE();
+            CATCOC_MMA(fa1, fb1, 0, 3)
+            slot2();
+            slot3();
+            CATCOC_FENCE();
+            CATCOC_MMA(fa0, fb0, 0, 0)
+            read_a(fa1, 1);
+            read_b1(fb1, sb, 1, 0);
+            CATCOC_FENCE();
+            CATCOC_MMA(fa0, fb0, 0, 1)
+            read_b1(fb1, sb, 1, 1);
+            read_b1(fb1, sb, 1, 2);
+            CATCOC_FENCE();
+            CATCOC_MMA(fa0, fb0, 0, 2)
+            read_b1(fb1, sb, 1, 3);
+            slot4();
+            CATCOC_FENCE();
+            CATCOC_MMA(fa0, fb0, 0, 3)
+        } else {
         CATCOC_MMA(fa1, fb1, 0, 0)
         read_a(fa0, 0);
         CATCOC_FENCE();
@@ -340,11 +366,12 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         CATCOC_FENCE();
         CATCOC_MMA(fa0, fb0, 0, 3)
         CATCOC_MMA(fa0, fb0, 1, 3)
+        }
     };
 #undef CATCOC_MMA
     auto nothing = [] {};
 
-    if constexpr (BM == 128) {
+    if constexpr (WM == 2) {
         // ---- 3 stages, copies run two k steps ahead (72 KiB LDS, two workgroups per CU) ----
         auto stA = [&](uint32_t s3) { return smem + s3 * A_STAGE; };
         auto stB = [&](uint32_t s3) { return smem + 3 * A_STAGE + s3 * B_STAGE; };
@@ -537,7 +564,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
     if constexpr (WM == 2) {
         if (kSlices > 1) {
             constexpr int DEVICE_SCOPE = 16;   // sc1
-            constexpr uint32_t TILE_WORDS = 128 * 256;
+            constexpr uint32_t TILE_WORDS = BM * 256;
             const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
                 (void *)(args.skPart + ((size_t)task * kSlices + slice) * TILE_WORDS), 0, (int)(TILE_WORDS * 4), 0x00020000);
 #pragma unroll
@@ -787,7 +814,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
         else stage_all([](float f) { return f32_to_f16_bits(f); });
         unsigned char *dwave = (unsigned char *)args.d + (((int64_t)(int32_t)out_row0 + wm * 32 * MB) * args.ldd + ti.col + wn * 128) * 2;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
+        for (int j = 0; j < 8 * MB; ++j) {
             if constexpr (RM) if (!(keptMb & (1u << (j >> 3)))) continue;   // rows 4j .. 4j+3 of the wave: 32-row block j / 8
             const uint32_t wrow = j * 4 + (lane >> 4), chunk = lane & 15;
             const v4i v = *(const v4i *)(st + wrow * 256 + ((chunk * 16) ^ (((wrow >> 2) & 1) << 7)));
@@ -875,15 +902,28 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             }
         }
         if (!summed) {
+            if constexpr (DT == DT_I8) {
+                // exact in 32-bit arithmetic: a = (a >> 16) * 65536 + (a & 0xffff), and 128 of either part add without overflow
+                int hi = 0, lo = 0;
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+                for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int nb = 0; nb < 4; ++nb)
+                    for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        if constexpr (DT == DT_I8) si += acc[mb][nb][r];
-                        else si += (double)getf(mb, nb, r);
-                    }
+                        for (int r = 0; r < 16; ++r) {
+                            const int a = acc[mb][nb][r];
+                            hi += a >> 16;
+                            lo += a & 0xffff;
+                        }
+                si = (long long)hi * 65536 + lo;
+            } else {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) si += (double)getf(mb, nb, r);
+            }
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) si += __shfl_xor(si, o, 64);
@@ -900,6 +940,57 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 
 }
 
+// One workgroup per tile, or per k slice of a tile.
+template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false>
+__global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<WM>::BYTES];
+    // A launch with few tiles can cut every tile's k range into kSlices pieces, one workgroup each (128-row tiles
+    // only): position `pos` of the launch order runs as kSlices workgroups that stay in the position's XCD column.
+    uint32_t pos = blockIdx.x + args.taskBase, slice = 0;   // (taskBase is zero for k-sliced launches)
+    const uint32_t kSlices = (WM == 2 && args.splitK > 1) ? args.splitK : 1u;
+    if (kSlices > 1) {
+        if ((args.sched.coreLoops & 7u) == 0) {
+            const uint32_t q = blockIdx.x >> 3;
+            slice = q % kSlices;
+            pos = (q / kSlices) * 8u + (blockIdx.x & 7u);
+        } else {
+            slice = blockIdx.x % kSlices;
+            pos = blockIdx.x / kSlices;
+        }
+    }
+    dma_tile<DT, WM, TB, RM, RG, TA, 2>(args, smem, pos, slice, kSlices, 0);
+}
+
+// Reduce-scatter launches of a single round of workgroups (no more tiles than the 512 slots of the GPU): every kept 128-row
+// tile runs as two 64-row workgroups.  A kept tile is the longest chain of such a launch (its main loop, then the peers'
+// partials from HBM) and nothing follows it, so the launch lasts as long as that chain; cut in two, each half streams half
+// the peers.  Launch order inside an XCD (workgroup id = 8 * j + xcd): j < 2 * kept tiles of the XCD -> kept tile j / 2, rows
+// 64 * (j & 1) ..; later j -> the other tiles in their usual order.  Requires the XCD-block order, the same number of kept
+// tiles on every XCD (keptPerXcd), whole tiles, plain operand layouts, one launch for all tasks.
+template <uint32_t DT>
+__global__ void __launch_bounds__(256, 2) gemm_dma_split_kept_kernel(const GemmArgs args, const uint32_t keptPerXcd)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<2>::BYTES];
+    const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    if (j < 2u * keptPerXcd) dma_tile<DT, 2, false, false, false, false, 1>(args, smem, (j >> 1) * 8u + x, 0, 1, (j & 1u) * 64u);
+    else dma_tile<DT, 2, false, false, false, false, 2>(args, smem, (j - keptPerXcd) * 8u + x, 0, 1, 0);
+}
+
+// Kept tiles per XCD when a launch qualifies for gemm_dma_split_kept_kernel, else 0: a whole reduce-scatter launch in the
+// XCD-block order, plain operand layouts, the kept rows exactly the kept rank's block with peers to stream, no more tiles
+// than one round of workgroups and at most 48 k steps per tile.  Measured with 512 tiles (W8A8, N = 4096): 16 / 28 / 40
+// k steps run 32 / 27 / 17 % faster split, 56 steps 5 % slower; two rounds of tiles (1024) 10 % slower.
+inline uint32_t split_kept_tiles(const GemmArgs &a, uint32_t kSteps)
+{
+    const SchedParams &s = a.sched;
+    if (s.m0 != 128 || a.splitK > 1 || a.taskBase != 0 || a.taskCount != 0 || (a.flags & (GF_LINEAR_ORDER | GF_ROW_MASK | GF_RAGGED)) ||
+        a.transA || a.transB || a.nPeers == 0 || a.keptBegin != a.keptRank * s.mRank || a.keptRows != s.mRank)
+        return 0;
+    if (s.coreLoops > 512u || kSteps > 48u) return 0;
+    return xcd_uniform_kept(s, a.keptRank);
+}
+
 // Launch of the 128-row geometry: one instantiation per operand layout (A as [m][k] or [k][m], B as [k][n] or [n][k]) and
 // for ragged problems; one workgroup per tile, or per k slice of a tile.
 template <uint32_t DT>
@@ -907,7 +998,12 @@ inline int launch_dma_128(const GemmArgs &args, hipStream_t s)
 {
     const dim3 grid(launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u)), block(256);
     switch ((args.transA ? 4 : 0) | (args.transB ? 2 : 0) | ((args.flags & GF_RAGGED) ? 1 : 0)) {
-        case 0: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false>), grid, block, 0, s, args); break;
+        case 0:
+            if (const uint32_t keptPerXcd = split_kept_tiles(args, args.K * (DT == DT_I8 ? 1u : 2u) / 64u))
+                hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT>), dim3(args.sched.coreLoops + 8u * keptPerXcd), block, 0, s, args, keptPerXcd);
+            else
+                hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false>), grid, block, 0, s, args);
+            break;
         case 1: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, true, false>), grid, block, 0, s, args); break;
         case 2: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, false, false>), grid, block, 0, s, args); break;
         case 3: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, true, false>), grid, block, 0, s, args); break;

@@ -468,6 +468,24 @@ CATCOC_HD void xcd_launch_tile(const SchedParams &s, uint32_t keptRank, uint32_t
     ti.wsRow = (stage * s.blockPerComm + b) * s.m0;
 }
 
+// Kept tiles of one XCD's block under the XCD-block order when all eight XCDs hold the same number (they are then the first
+// positions of every XCD), else 0.
+inline uint32_t xcd_uniform_kept(const SchedParams &s, uint32_t keptRank)
+{
+    if (!s.xOk || s.op != OP_REDUCE_SCATTER || s.P <= 1 || (s.coreLoops & 7u) != 0) return 0;
+    uint32_t per = 0;
+    for (uint32_t x = 0; x < 8; ++x) {
+        const uint32_t rp = x >> s.xCxLog;
+        const uint32_t lo = keptRank * s.loopsM, hi = lo + s.loopsM, up = (1u << s.xRxLog) - 1u;
+        const uint32_t i0 = umin(lo > rp ? (lo - rp + up) >> s.xRxLog : 0u, s.xRowsPer);
+        const uint32_t i1 = umin(hi > rp ? (hi - rp + up) >> s.xRxLog : 0u, s.xRowsPer);
+        const uint32_t k = (i1 - i0) * s.xColsPer;
+        if (x == 0) per = k;
+        else if (k != per) return 0;
+    }
+    return per;
+}
+
 // Workgroup -> task and tile of a launch of the direct-to-LDS kernels; false past the end of the launch.
 CATCOC_HD bool launch_tile(const SchedParams &s, uint32_t wg, bool linear, uint32_t keptRank, uint32_t &task, TileInfo &ti);
 

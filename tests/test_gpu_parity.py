@@ -514,6 +514,38 @@ def test_float_reduce_scatter(dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+def test_float_single_round_launch_splits_kept_tiles(dtype):
+    # at most 512 tiles and short k: every kept tile runs as two 64-row workgroups (a second tile body inside the kernel);
+    # kept block, accumulators of every tile, checksums of the other ranks' tiles
+    _need_gpu()
+    import ctypes as C
+    M, N, K, P, rank = 4096, 2048, 640, 8, 3          # 256 tiles, 20 k steps
+    rng = np.random.default_rng(28)
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    part, want = oracle.matmul_reduce(A, B, dtype, rank * rows, rows, peers, want_partial=True)
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    so = L.load()
+    ntasks = so.catcoc_get_task_count(L.MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+    cs = torch.zeros(ntasks, dtype=torch.float64, device=DEV)
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    for _ in range(2):
+        out = ops.matmul_reduce_scatter(dev16(A, dtype), dev16(B, dtype), [dev(p) for p in peers], rank, P, checksum=cs, acc_dump=dump)
+        torch.cuda.synchronize()
+    _check_float(host16(out), want, part[rank * rows:(rank + 1) * rows] + sum(peers), dtype, K)
+    assert np.abs(dump.cpu().numpy() - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
+    tr, row, col, ws = (C.c_uint32() for _ in range(4))
+    for task in range(ntasks):
+        so.catcoc_task_tile(L.MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row), C.byref(col), C.byref(ws))
+        blk = part[row.value:row.value + 128, col.value:col.value + 256]
+        want_cs = 0.0 if tr.value == rank else float(blk.astype(np.float64).sum())
+        assert abs(float(cs[task]) - want_cs) <= 1e-2 * max(1.0, np.abs(blk).sum()), task
+
+
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
 def test_float_ragged_problems_on_many_tiles(dtype):
     # full tiles on the direct-to-LDS kernel, ragged ones on the bounds-checked kernel, in two launches
     _need_gpu()
