@@ -46,10 +46,28 @@ def cpu_baseline(M, N, K, P, rank, repeats):
         run()
         ts.append(time.perf_counter() - t0)
     best = min(ts)
-    return {"value": 2.0 * M * N * K / best / 1e12, "unit": "TOPS", "cores": oracle.num_threads(), "kind": "port",
-            "sample": "full workload (M=%d,K=%d,N=%d,P=%d), 1 warm-up + %d timed runs, best %.3f s, mean %.3f s; "
-                      "OpenMP over rows, gcc -O3 -march=native -ffp-contract=off" % (M, K, N, P, repeats, best,
-                                                                                    sum(ts) / len(ts))}
+    out = {"value": 2.0 * M * N * K / best / 1e12, "unit": "TOPS", "cores": oracle.num_threads(), "kind": "port",
+           "sample": "full workload (M=%d,K=%d,N=%d,P=%d), 1 warm-up + %d timed runs, best %.3f s, mean %.3f s; "
+                     "OpenMP over rows, gcc -O3 -march=native -ffp-contract=off" % (M, K, N, P, repeats, best,
+                                                                                   sum(ts) / len(ts))}
+    # the reference's own golden (Catlass::golden::QuantMatmul, 3rdparty/catlass/examples/common/golden/matmul.hpp:274-302,
+    # compiled from its sources into oracle/_ref where that was possible): the literal triple loop, one core, on a
+    # down-scaled shape of the same K
+    ref = oracle.ref_golden()
+    if ref is not None:
+        import ctypes as C
+        m1, n1 = 256, 512
+        want = np.empty((m1, n1), np.float32)
+        a1, b1 = np.ascontiguousarray(x1[:m1]), np.ascontiguousarray(x2[:, :n1])
+        p_ = lambda a: a.ctypes.data_as(C.c_void_p)
+        t0 = time.perf_counter()
+        ref.ref_quant_matmul(C.c_uint32(m1), C.c_uint32(n1), C.c_uint32(K), p_(a1), p_(b1), p_(np.ascontiguousarray(s2[:n1])),
+                             p_(np.ascontiguousarray(s1[:m1])), p_(want))
+        dt = time.perf_counter() - t0
+        out["reference_single_core"] = {"value": 2.0 * m1 * n1 * K / dt / 1e12, "unit": "TOPS", "cores": 1, "kind": "reference",
+                                        "sample": "Catlass::golden::QuantMatmul on M=%d,K=%d,N=%d (GEMM + dequant only), one run, "
+                                                  "%.3f s" % (m1, K, n1, dt)}
+    return out
 
 
 def decode_sweep(args, torch, L, ops, dev):
