@@ -97,6 +97,12 @@ typedef void (*CatcocKernelFuncPtr)(void *stream, uint64_t fftsAddr, uint8_t *a,
 #define CATCOC_FLAG_REDUCE_INT32 0x4u
 /* Keep the linear workgroup -> task order (no XCD-aware chunking). */
 #define CATCOC_FLAG_LINEAR_ORDER 0x8u
+/* Reduce-scatter launches of one round of workgroups (at most 512 tiles of 128x256 with at most 64 k steps of 64 bytes,
+ * or fewer than 256 tiles) run every kept tile as two 64-row workgroups, which halves the chain of peer partials a
+ * workgroup adds; the library decides by those two numbers.  KEPT_WHOLE never splits, KEPT_SPLIT splits whenever the launch allows it (whole
+ * tiles, A as [m,k], XCD-aware order): tuning knobs like the tiling's, results are bit-identical either way. */
+#define CATCOC_FLAG_KEPT_WHOLE 0x10u
+#define CATCOC_FLAG_KEPT_SPLIT 0x20u
 
 /* Replaces the reference's `symmetricPtr` workspace + shmem_my_pe()/shmem_n_pes()
  * (examples/dynamic_tiling/impl/kernel/matmul_reduce_scatter.h:155-156): which
@@ -358,9 +364,9 @@ CATCOC_API uint32_t catcoc_task_tiles(int commType, const CocTilingParams *tilin
                                       uint32_t *wsRow);
 /* The task workgroup `wg` of a launch runs: an XCD-aware order with the kept rank's tiles first (they are the
  * long ones).  A bijection on [0, task count);
- * 0xffffffff for wg out of range or rejected arguments.  (A reduce-scatter launch of at most 512 tiles with short
- * k runs every kept tile as two 64-row workgroups, placed first in the same order; this function still describes
- * the order by tile.)  No counterpart in the reference, where AI core i
+ * 0xffffffff for wg out of range or rejected arguments.  (A reduce-scatter launch that splits its kept tiles, see
+ * CATCOC_FLAG_KEPT_SPLIT, runs each as two 64-row workgroups placed first in the same order; this function still
+ * describes the order by tile.)  No counterpart in the reference, where AI core i
  * simply runs tasks i, i + BLOCK_NUM, ... (quant_matmul_reduce_scatter.hpp:166-170). */
 CATCOC_API uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
                                        uint32_t wg);

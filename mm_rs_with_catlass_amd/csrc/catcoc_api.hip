@@ -161,6 +161,8 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
         a.flags |= GF_REDUCE_INT32;
     }
     if (d->flags & CATCOC_FLAG_LINEAR_ORDER) a.flags |= GF_LINEAR_ORDER;
+    if (d->flags & CATCOC_FLAG_KEPT_WHOLE) a.flags |= GF_KEPT_WHOLE;
+    if (d->flags & CATCOC_FLAG_KEPT_SPLIT) a.flags |= GF_KEPT_SPLIT;
     if (plan.dma && plan.edge) a.flags |= GF_RAGGED;
 
     // kept rows

@@ -18,6 +18,8 @@ enum : uint32_t {
     GF_ROW_MASK = 1u << 3,        // kept rows [keptBegin, +keptRows) are whole 32-row blocks that need not line up with tiles: the
                                   // epilogue works per 32-row block, and `checksum` takes the rows that are not kept per 128 x 128
                                   // block, index (row / 128) * (N / 128) + col / 128
+    GF_KEPT_WHOLE = 1u << 5,      // never run kept tiles as two 64-row workgroups
+    GF_KEPT_SPLIT = 1u << 6,      // do so whenever the launch allows it (default: by tile count and k length)
     GF_RAGGED = 1u << 4,          // the last tile row of a rank and / or the last tile column are not full: such tiles are computed as
                                   // whole tiles moved up / left so that they end at the edge (they overlap their neighbours, whose
                                   // values they reproduce bit for bit); sums and workspace stores leave the overlap out

@@ -92,7 +92,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     static_assert(!RG || (WM == 2 && !RM), "ragged mode exists for the 128-row kernel");
     static_assert(!TA || (WM == 2 && !RM), "transposed A exists for the 128-row kernel");
     static_assert(WM == 2 || WM == 4, "supported geometries");
-    static_assert(MB == 2 || (MB == 1 && WM == 2 && !RM && !RG && !TA), "64-row tiles exist for the plain four-wave geometry");
+    static_assert(MB == 2 || (MB == 1 && WM == 2 && !RM && !RG && !TA), "64-row tiles exist for the four-wave geometry with A as [m,k]");
     using Acc = typename AccOf<DT>::type;
     constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
     constexpr int NW = 2 * WM;          // waves
@@ -967,27 +967,30 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
 // partials from HBM) and nothing follows it, so the launch lasts as long as that chain; cut in two, each half streams half
 // the peers.  Launch order inside an XCD (workgroup id = 8 * j + xcd): j < 2 * kept tiles of the XCD -> kept tile j / 2, rows
 // 64 * (j & 1) ..; later j -> the other tiles in their usual order.  Requires the XCD-block order, the same number of kept
-// tiles on every XCD (keptPerXcd), whole tiles, plain operand layouts, one launch for all tasks.
-template <uint32_t DT>
+// tiles on every XCD (keptPerXcd), whole tiles, A as [m,k], one launch for all tasks.
+template <uint32_t DT, bool TB>
 __global__ void __launch_bounds__(256, 2) gemm_dma_split_kept_kernel(const GemmArgs args, const uint32_t keptPerXcd)
 {
     __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<2>::BYTES];
     const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
-    if (j < 2u * keptPerXcd) dma_tile<DT, 2, false, false, false, false, 1>(args, smem, (j >> 1) * 8u + x, 0, 1, (j & 1u) * 64u);
-    else dma_tile<DT, 2, false, false, false, false, 2>(args, smem, (j - keptPerXcd) * 8u + x, 0, 1, 0);
+    if (j < 2u * keptPerXcd) dma_tile<DT, 2, TB, false, false, false, 1>(args, smem, (j >> 1) * 8u + x, 0, 1, (j & 1u) * 64u);
+    else dma_tile<DT, 2, TB, false, false, false, 2>(args, smem, (j - keptPerXcd) * 8u + x, 0, 1, 0);
 }
 
 // Kept tiles per XCD when a launch qualifies for gemm_dma_split_kept_kernel, else 0: a whole reduce-scatter launch in the
-// XCD-block order, plain operand layouts, the kept rows exactly the kept rank's block with peers to stream, no more tiles
-// than one round of workgroups and at most 48 k steps per tile.  Measured with 512 tiles (W8A8, N = 4096): 16 / 28 / 40
-// k steps run 32 / 27 / 17 % faster split, 56 steps 5 % slower; two rounds of tiles (1024) 10 % slower.
+// XCD-block order, A as [m,k], the kept rows exactly the kept rank's block with peers to stream, and by default either
+// fewer tiles than CUs or at most one round of workgroups (512 tiles) with at most 64 k steps per tile.  Measured with
+// the two variants alternating launch by launch (W8A8, N = 4096, whole -> split, us): 512 tiles with 28 / 40 / 56 / 72 /
+// 80 / 112 k steps 54.4 -> 40.5 / 65.7 -> 54.5 / 79.6 -> 73.7 / 92.3 -> 91.8 / 102.9 -> 106.2 / 128.7 -> 140.9; 128 tiles
+// with 112 steps 67.3 -> 49.8; 768 tiles 59.3 -> 59.1; 1024 tiles 74.8 -> 83.3.  GF_KEPT_WHOLE / GF_KEPT_SPLIT override.
 inline uint32_t split_kept_tiles(const GemmArgs &a, uint32_t kSteps)
 {
     const SchedParams &s = a.sched;
     if (s.m0 != 128 || a.splitK > 1 || a.taskBase != 0 || a.taskCount != 0 || (a.flags & (GF_LINEAR_ORDER | GF_ROW_MASK | GF_RAGGED)) ||
-        a.transA || a.transB || a.nPeers == 0 || a.keptBegin != a.keptRank * s.mRank || a.keptRows != s.mRank)
+        a.transA || a.nPeers == 0 || a.keptBegin != a.keptRank * s.mRank || a.keptRows != s.mRank)
         return 0;
-    if (s.coreLoops > 512u || kSteps > 48u) return 0;
+    if (a.flags & GF_KEPT_WHOLE) return 0;
+    if (!(a.flags & GF_KEPT_SPLIT) && !(s.coreLoops < 256u || (s.coreLoops <= 512u && kSteps <= 64u))) return 0;
     return xcd_uniform_kept(s, a.keptRank);
 }
 
@@ -1000,12 +1003,17 @@ inline int launch_dma_128(const GemmArgs &args, hipStream_t s)
     switch ((args.transA ? 4 : 0) | (args.transB ? 2 : 0) | ((args.flags & GF_RAGGED) ? 1 : 0)) {
         case 0:
             if (const uint32_t keptPerXcd = split_kept_tiles(args, args.K * (DT == DT_I8 ? 1u : 2u) / 64u))
-                hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT>), dim3(args.sched.coreLoops + 8u * keptPerXcd), block, 0, s, args, keptPerXcd);
+                hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT, false>), dim3(args.sched.coreLoops + 8u * keptPerXcd), block, 0, s, args, keptPerXcd);
             else
                 hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false>), grid, block, 0, s, args);
             break;
         case 1: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, true, false>), grid, block, 0, s, args); break;
-        case 2: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, false, false>), grid, block, 0, s, args); break;
+        case 2:
+            if (const uint32_t keptPerXcd = split_kept_tiles(args, args.K * (DT == DT_I8 ? 1u : 2u) / 64u))
+                hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT, true>), dim3(args.sched.coreLoops + 8u * keptPerXcd), block, 0, s, args, keptPerXcd);
+            else
+                hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, false, false>), grid, block, 0, s, args);
+            break;
         case 3: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, true, false>), grid, block, 0, s, args); break;
         case 4: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, true>), grid, block, 0, s, args); break;
         case 5: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, true, true>), grid, block, 0, s, args); break;

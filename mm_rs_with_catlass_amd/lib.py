@@ -22,6 +22,8 @@ OUTBOUND_CHECKSUM = 0
 OUTBOUND_STORE = 1
 FLAG_REDUCE_INT32 = 4
 FLAG_LINEAR_ORDER = 8
+FLAG_KEPT_WHOLE = 0x10
+FLAG_KEPT_SPLIT = 0x20
 
 
 class CatcocError(RuntimeError):

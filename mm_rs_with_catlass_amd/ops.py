@@ -88,6 +88,11 @@ def _task_count(comm_type, t, d):
     return n
 
 
+def _kept_flag(kept_split):
+    """kept_split: None = the library decides, False = kept tiles whole, True = two 64-row workgroups where allowed."""
+    return 0 if kept_split is None else (_l.FLAG_KEPT_SPLIT if kept_split else _l.FLAG_KEPT_WHOLE)
+
+
 def _attach_workspace(d, workspace, split_k):
     """Optional scratch for k-sliced launches (kslice_plan() says how large) and the caller's own slice count."""
     d.splitK = split_k
@@ -109,7 +114,7 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
                                         out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
                                         reduce_int32=False, outbound=None, checksum=None, acc_dump=None,
                                         c_accum=None, block_num=0, stages=0, swizzle=None, linear_order=False,
-                                        out=None, workspace=None, split_k=0, trans_a=False):
+                                        out=None, workspace=None, split_k=0, trans_a=False, kept_split=None):
     """Validate and bind the arguments once; returns (launch, out) where launch() enqueues one call of
     catcoc_launch_quant_matmul_reduce_scatter on torch's current stream (for launch-rate-sensitive loops)."""
     _check_rank(rank, rank_size)
@@ -135,7 +140,7 @@ def prepare_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, p
     if (t.m, t.k, t.n) != (m, k, n):
         _fail("tiling says m,k,n = %d,%d,%d; the operands say %d,%d,%d", t.m, t.k, t.n, m, k, n)
     flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_REDUCE_INT32 if reduce_int32 else 0) | \
-        (_l.FLAG_LINEAR_ORDER if linear_order else 0)
+        (_l.FLAG_LINEAR_ORDER if linear_order else 0) | _kept_flag(kept_split)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
     _attach_workspace(d, workspace, split_k)
     if checksum is not None:
@@ -160,7 +165,7 @@ def quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
                                 out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0,
                                 reduce_int32=False, outbound=None, checksum=None, acc_dump=None, c_accum=None,
                                 block_num=0, stages=0, swizzle=None, linear_order=False, out=None, workspace=None,
-                                split_k=0, trans_a=False):
+                                split_k=0, trans_a=False, kept_split=None):
     """W8A8 matmul -> reduce-scatter share of one rank.
 
     x1 [m,k] int8 ([k,m] with trans_a), x2 [k,n] int8 ([n,k] with trans_b), scale_x1 [m] fp32 per token, scale_x2 [n] fp32 per
@@ -172,7 +177,7 @@ def quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
     launch, out = prepare_quant_matmul_reduce_scatter(
         x1, x2, scale_x1, scale_x2, bias, peers, rank, rank_size, out_dtype, tiling, trans_b, peer_row_offset,
         reduce_int32, outbound, checksum, acc_dump, c_accum, block_num, stages, swizzle, linear_order, out, workspace, split_k,
-        trans_a)
+        trans_a, kept_split)
     launch()
     _l.check()
     return out
@@ -246,7 +251,8 @@ def quant_matmul_splitk(*args, **kw):
 
 
 def _float_op(comm_type, a, b, c_shape, peers, rank, rank_size, tiling, trans_a, trans_b, peer_row_offset, outbound,
-              checksum, acc_dump, block_num, stages, swizzle, linear_order, out, m_for_tiling, workspace=None, split_k=0):
+              checksum, acc_dump, block_num, stages, swizzle, linear_order, out, m_for_tiling, workspace=None, split_k=0,
+              kept_split=None):
     if a.dtype not in _TORCH_TO_DT or b.dtype != a.dtype:
         raise _l.CatcocError("a and b must both be float16 or both bfloat16")
     _check_rank(rank, rank_size)
@@ -274,7 +280,7 @@ def _float_op(comm_type, a, b, c_shape, peers, rank, rank_size, tiling, trans_a,
     t = tiling if tiling is not None else default_tiling(m_for_tiling, k, n, rank_size, m0=0, n0=0, k0=0)
     if (t.m, t.k, t.n) != (m_for_tiling, k, n):
         _fail("tiling says m,k,n = %d,%d,%d; the operands say %d,%d,%d", t.m, t.k, t.n, m_for_tiling, k, n)
-    flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_LINEAR_ORDER if linear_order else 0)
+    flags = (_l.OUTBOUND_STORE if outbound is not None else 0) | (_l.FLAG_LINEAR_ORDER if linear_order else 0) | _kept_flag(kept_split)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, flags, block_num, stages, swizzle, outbound, checksum, acc_dump)
     _attach_workspace(d, workspace, split_k)
     if checksum is not None:
@@ -295,12 +301,12 @@ def _float_op(comm_type, a, b, c_shape, peers, rank, rank_size, tiling, trans_a,
 
 def matmul_reduce_scatter(a, b, peers=(), rank=0, rank_size=1, tiling=None, trans_a=False, trans_b=False,
                           peer_row_offset=0, outbound=None, checksum=None, acc_dump=None, block_num=0, stages=0,
-                          swizzle=None, linear_order=False, out=None, workspace=None, split_k=0):
+                          swizzle=None, linear_order=False, out=None, workspace=None, split_k=0, kept_split=None):
     """fp16/bf16 matmul -> reduce-scatter share: a [m,k], b [k,n], peers fp32; returns [m/rank_size, n]."""
     m = a.shape[1] if trans_a else a.shape[0]
     return _float_op(_l.MATMUL_REDUCE_SCATTER, a, b, lambda n: (m // max(rank_size, 1), n), peers, rank, rank_size,
                      tiling, trans_a, trans_b, peer_row_offset, outbound, checksum, acc_dump, block_num, stages,
-                     swizzle, linear_order, out, m, workspace, split_k)
+                     swizzle, linear_order, out, m, workspace, split_k, kept_split)
 
 
 def matmul_allreduce(a, b, peers=(), rank=0, rank_size=1, tiling=None, trans_a=False, trans_b=False,

@@ -187,6 +187,34 @@ def test_quant_rs_ragged_problem_on_many_tiles(case):
     assert seen_ragged > 0 and seen_full >= 64 and r["ntasks"] <= 256
 
 
+@pytest.mark.parametrize("tb", [False, True])
+def test_quant_rs_kept_tiles_whole_or_split_give_the_same_bits(tb):
+    # CATCOC_FLAG_KEPT_WHOLE / CATCOC_FLAG_KEPT_SPLIT are tuning knobs: output, kept accumulators and checksums must not change
+    _need_gpu()
+    import ctypes as C
+    M, N, K, P, rank = 8192, 1024, 448, 8, 5          # 256 tiles; also forced on 1024 tiles below
+    for (M, N) in ((8192, 1024), (8192, 4096)):
+        g = torch.Generator(device=DEV).manual_seed(11)
+        x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
+        x2 = torch.randint(-127, 128, (N, K) if tb else (K, N), dtype=torch.int8, device=DEV, generator=g)
+        s1 = torch.empty(M, device=DEV).uniform_(0.005, 0.02, generator=g)
+        s2 = torch.empty(N, device=DEV).uniform_(0.001, 0.01, generator=g)
+        peers = [torch.randn((M // P, N), device=DEV, generator=g) for _ in range(P - 1)]
+        t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+        d = L.make_desc(rank, P, [16] * (P - 1))
+        ntasks = L.load().catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+        res = []
+        for ks in (False, True, None):
+            cs = torch.zeros(ntasks, dtype=torch.int64, device=DEV)
+            ca = torch.zeros((M // P, N), dtype=torch.int32, device=DEV)
+            out = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, rank, P, trans_b=tb, checksum=cs, c_accum=ca, kept_split=ks)
+            torch.cuda.synchronize()
+            res.append((out.view(torch.int16).clone(), cs, ca))
+        for r in res[1:]:
+            assert torch.equal(res[0][0], r[0]) and torch.equal(res[0][1], r[1]) and torch.equal(res[0][2], r[2])
+        assert int(res[0][1].ne(0).sum()) >= ntasks * 7 // 8 - 2
+
+
 @pytest.mark.parametrize("shape", [(32, 129, 100), (24, 7, 3), (4 * 23, 45, 68), (4, 128, 512)])
 def test_quant_rs_general_shapes(shape):
     # K not a multiple of 16 or N not a multiple of 4: the general kernel (incl. the reference's own
