@@ -370,6 +370,11 @@ CATCOC_API uint32_t catcoc_task_tiles(int commType, const CocTilingParams *tilin
  * simply runs tasks i, i + BLOCK_NUM, ... (quant_matmul_reduce_scatter.hpp:166-170). */
 CATCOC_API uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
                                        uint32_t wg);
+/* How many kept tiles a launch of this shape would run as two 64-row workgroups each (see CATCOC_FLAG_KEPT_SPLIT;
+ * 0 = none: the launch then has one workgroup per task, else that many workgroups more).  For tools that size or
+ * reason about the grid.  No counterpart in the reference. */
+CATCOC_API uint32_t catcoc_kept_split_tiles(int commType, int dataType, const CocTilingParams *tiling,
+                                            const CatcocSymmetricDesc *desc, uint32_t transA, uint32_t transB);
 /* The same with the tile: what workgroup `wg` of the launch computes, exactly as the kernel works it out (the
  * large-tile kernels take a division-free route through constants prepared per launch; this entry point is how
  * tests compare that route with catcoc_launch_task + catcoc_task_tile).  Returns 0 past the end of the launch. */

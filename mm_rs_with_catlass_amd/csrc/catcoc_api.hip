@@ -913,6 +913,20 @@ uint32_t catcoc_launch_task(int commType, const CocTilingParams *tiling, const C
     return launch_task(s, wg, (p.args.flags & GF_LINEAR_ORDER) != 0, p.args.keptRank);
 }
 
+uint32_t catcoc_kept_split_tiles(int commType, int dataType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
+                                 uint32_t transA, uint32_t transB)
+{
+    Plan p;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
+    d = *desc;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    if (make_plan(commType, dataType, tiling, &d, transA, transB, p)) return 0;
+    ok();
+    if (!p.dma || p.args.sched.m0 != 128) return 0;
+    return 8u * split_kept_tiles(p.args, p.args.K * elem_size(p.dtype) / 64u);
+}
+
 uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags)
 {
     return workgroup_task(wg, tasks, (flags & CATCOC_FLAG_LINEAR_ORDER) != 0);

@@ -529,3 +529,34 @@ def test_task_tiles_batch_query_equals_single_queries(so):
         assert tuple(a[task] for a in arr) == tuple(x.value for x in one)
         assert tuple(a[task] for a in arr) == (lambda r: (r[0], r[3], r[4], r[5]))(oracle.rs_task(8192, 4096, 8, 128, 256, 20, 10, 2, task))
     assert so.catcoc_task_tiles(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), 1000, 100, None, arr[1], None, None) == 24
+
+
+def test_kept_split_choice_by_tile_count_and_k_length():
+    # which reduce-scatter launches run their kept tiles as two 64-row workgroups (catcoc_kept_split_tiles): fewer than 256
+    # tiles, or up to 512 tiles with up to 64 k steps of 64 bytes; whole tiles, A as [m,k], XCD-block order; flags override
+    from mm_rs_with_catlass_amd import ops
+    so = L.load()
+
+    def split(comm, dt, m, k, n, p, flags=0, ta=0, tb=0, rank=0):
+        t = ops.default_tiling(m, k, n, p, m0=0, n0=0, k0=0)
+        d = L.make_desc(rank, p, [16] * (p - 1))
+        d.flags = flags
+        r = so.catcoc_kept_split_tiles(comm, dt, C.byref(t), C.byref(d), ta, tb)
+        L.check()
+        return r
+    Q, RS = L.QUANT_MATMUL_REDUCE_SCATTER, L.MATMUL_REDUCE_SCATTER
+    assert split(Q, L.INT8, 8192, 1792, 4096, 8) == 0                 # config 4: 1024 tiles, two rounds
+    assert split(Q, L.INT8, 8192, 1792, 4096, 8, L.FLAG_KEPT_SPLIT) == 128
+    assert split(Q, L.INT8, 4096, 1792, 4096, 8) == 64                # 512 tiles, 28 k steps
+    assert split(Q, L.INT8, 4096, 1792, 4096, 8, tb=1) == 64          # either layout of B
+    assert split(Q, L.INT8, 4096, 1792, 4096, 8, ta=1) == 0           # A as [k,m]: whole tiles only
+    assert split(Q, L.INT8, 4096, 1792, 4096, 8, L.FLAG_KEPT_WHOLE) == 0
+    assert split(Q, L.INT8, 4096, 1792, 4096, 8, L.FLAG_LINEAR_ORDER) == 0
+    assert split(Q, L.INT8, 4096, 4096, 4096, 8) == 64                # 64 k steps
+    assert split(Q, L.INT8, 4096, 4160, 4096, 8) == 0                 # 65
+    assert split(Q, L.INT8, 1024, 7168, 4096, 8) == 16                # 128 tiles: fewer than CUs, any k
+    assert split(RS, L.FP16, 4096, 1792, 4096, 8) == 64               # config 3: 512 tiles, 56 k steps
+    assert split(RS, L.FP16, 4096, 2112, 4096, 8) == 0                # 66 k steps
+    assert split(RS, L.FP16, 8 * 296, 512, 1344, 8) == 0              # ragged problems keep whole tiles
+    assert split(L.MATMUL_ALLREDUCE, L.FP16, 1024, 512, 1024, 2) == 0 # no kept-rank block to split
+    assert split(Q, L.INT8, 4096, 1792, 4096, 1) == 0                 # no peers to stream
