@@ -79,12 +79,12 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 //   128-row tile: three A stages (8 KiB each), then three B stages (16 KiB each)            = 72 KiB
 //   256-row tile: two A pair buffers (32 KiB each), then four B stages (16 KiB each)         = 128 KiB
 // (a 64-row tile of the four-wave geometry uses the first 60 KiB of the 72)
-template <int WM> struct DmaPool { static constexpr int BYTES = (WM == 4) ? (4 * 256 * 64 + 4 * 64 * 256) : 3 * (128 * 64 + 64 * 256); };
+template <int WM, int NS = 3> struct DmaPool { static constexpr int BYTES = (WM == 4) ? (4 * 256 * 64 + 4 * 64 * 256) : NS * (128 * 64 + 64 * 256); };
 
 // One tile (or one k slice of a tile) of the launch: position `pos` of the launch order, in the caller's LDS pool.
 // MB = 32-row blocks per wave (2; 1 = a 64-row tile, four-wave geometry only); subRow = first row of a 64-row tile inside
 // its 128-row tile of the schedule.
-template <uint32_t DT, int WM, bool TB, bool RM, bool RG, bool TA, int MB>
+template <uint32_t DT, int WM, bool TB, bool RM, bool RG, bool TA, int MB, int NS = 3, bool PP = false>
 __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *smem, uint32_t pos, uint32_t slice, uint32_t kSlices,
                                          uint32_t subRow)
 {
@@ -92,6 +92,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     static_assert(!RG || (WM == 2 && !RM), "ragged mode exists for the 128-row kernel");
     static_assert(!TA || (WM == 2 && !RM), "transposed A exists for the 128-row kernel");
     static_assert(WM == 2 || WM == 4, "supported geometries");
+    static_assert(NS == 3 || (WM == 2 && NS >= 3 && NS <= 8), "deeper rings exist for the 128-row kernel");
     static_assert(MB == 2 || (MB == 1 && WM == 2 && !RM && !RG && !TA), "64-row tiles exist for the four-wave geometry with A as [m,k]");
     using Acc = typename AccOf<DT>::type;
     constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
@@ -102,7 +103,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     constexpr int A_DMA = BM / 16 / NW;  // 1 KiB copies per wave per stage
     constexpr int B_DMA = 16 / NW;
     constexpr int STEP_DMA = A_DMA + B_DMA;
-    constexpr int POOL = DmaPool<WM>::BYTES;
+    constexpr int POOL = DmaPool<WM, NS>::BYTES;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -372,11 +373,31 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     auto nothing = [] {};
 
     if constexpr (WM == 2) {
-        // ---- 3 stages, copies run two k steps ahead (72 KiB LDS, two workgroups per CU) ----
-        auto stA = [&](uint32_t s3) { return smem + s3 * A_STAGE; };
-        auto stB = [&](uint32_t s3) { return smem + 3 * A_STAGE + s3 * B_STAGE; };
-        auto offA = [&](uint32_t s3) { return s3 * A_STAGE; };
-        auto offB = [&](uint32_t s3) { return 3 * A_STAGE + s3 * B_STAGE; };
+        // ---- NS stages, copies run NS - 1 k steps ahead.  NS = 3: 72 KiB LDS, two workgroups per CU, for operands that come
+        // out of L2 or the Infinity Cache.  NS = 6: 144 KiB, one workgroup per CU, 120 KiB in flight per CU: for launches of at
+        // most one workgroup per CU anyway, whose operands stream from HBM (two steps ahead do not cover that latency) ----
+        auto stA = [&](uint32_t st) { return smem + st * A_STAGE; };
+        auto stB = [&](uint32_t st) { return smem + NS * A_STAGE + st * B_STAGE; };
+        auto offA = [&](uint32_t st) { return st * A_STAGE; };
+        auto offB = [&](uint32_t st) { return NS * A_STAGE + st * B_STAGE; };
+        // wait until at most r whole steps of copies (the youngest) are outstanding, r < NS - 1
+        auto wait_steps = [&](uint32_t r) {
+            if constexpr (NS == 3) {
+                if (r) CATCOC_WAIT_VMCNT(STEP_DMA);
+                else CATCOC_WAIT_VMCNT(0);
+            } else {
+                switch (r) {
+                    case 0: CATCOC_WAIT_VMCNT(0); break;
+                    case 1: CATCOC_WAIT_VMCNT(STEP_DMA); break;
+                    case 2: CATCOC_WAIT_VMCNT(2 * STEP_DMA); break;
+                    case 3: CATCOC_WAIT_VMCNT(3 * STEP_DMA); break;
+                    case 4: CATCOC_WAIT_VMCNT((NS > 5 ? 4 : 0) * STEP_DMA); break;
+                    case 5: CATCOC_WAIT_VMCNT((NS > 6 ? 5 : 0) * STEP_DMA); break;
+                    default: CATCOC_WAIT_VMCNT((NS > 7 ? 6 : 0) * STEP_DMA); break;
+                }
+            }
+        };
+        static_assert((NS - 2) * STEP_DMA <= 63, "the wait counter holds 63");
         const uint32_t a_lds = (wm * 32 * MB + c32) * 64;
         const uint32_t a_sw = (c32 >> 2) & 3;
         // A as [k][m]: the transposing reads of B, with this wave's 32-row blocks in place of 32-column blocks
@@ -414,19 +435,18 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                 }
             }
         };
-        issue_a(offA(0));
-        issue_b(offB(0));
-        if (nk > 1) {
-            issue_a(offA(1));
-            issue_b(offB(1));
-        }
+#pragma unroll
+        for (int st = 0; st < NS - 1; ++st)
+            if (nk > (uint32_t)st) {
+                issue_a(offA(st));
+                issue_b(offB(st));
+            }
         // step 0 (peeled: no MFMAs pending yet)
-        if (nk > 1) CATCOC_WAIT_VMCNT(STEP_DMA);
-        else CATCOC_WAIT_VMCNT(0);
+        wait_steps(umin(NS - 2, nk - 1));
         barrier_keep_vmem();
-        if (nk > 2) {
-            issue_a(offA(2));
-            issue_b(offB(2));
+        if (nk > NS - 1) {
+            issue_a(offA(NS - 1));
+            issue_b(offB(NS - 1));
         }
         load_a(fa0, stA(0), 0);
         load_b(fb0, stB(0), 0);
@@ -435,24 +455,23 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
         CATCOC_FENCE();
         mma(fa0, fb0);
         CATCOC_FENCE();
-        // step kt reads stage kt % 3 and refills stage (kt + 2) % 3, which every wave left at the barrier
+        // step kt reads stage kt % NS and refills stage (kt - 1) % NS, which every wave left at the barrier
         uint32_t kt = 1, cur = 1, nxt = 0;
         auto step = [&](bool more) {
             const unsigned char *sa = stA(cur);
             sched_step([&](v4i (&af)[MB], int kk) { load_a(af, sa, kk); }, stB(cur),
                        [&] { if (more) issue_a(offA(nxt)); }, [&] { if (more) issue_b(offB(nxt)); }, nothing, nothing);
             ++kt;
-            cur = cur == 2 ? 0 : cur + 1;
-            nxt = nxt == 2 ? 0 : nxt + 1;
+            cur = cur == NS - 1 ? 0 : cur + 1;
+            nxt = nxt == NS - 1 ? 0 : nxt + 1;
         };
-        while (kt + 2 < nk) {
-            CATCOC_WAIT_VMCNT(STEP_DMA);
+        while (kt + (NS - 1) < nk) {
+            CATCOC_WAIT_VMCNT((NS - 2) * STEP_DMA);
             barrier_keep_vmem();
             step(true);
         }
         while (kt < nk) {
-            if (kt + 1 < nk) CATCOC_WAIT_VMCNT(STEP_DMA);
-            else CATCOC_WAIT_VMCNT(0);
+            wait_steps(nk - 1 - kt);
             barrier_keep_vmem();
             step(false);
         }
@@ -763,6 +782,93 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                 }
         }
 
+        if constexpr (PP) {
+            // One workgroup per CU (the deep ring): few tiles, so few kept tiles, and their peer partials are bound by memory
+            // latency, not bandwidth.  Fetched in accumulator layout (64 four-byte loads per 32-row block and peer) a wave
+            // cannot have more than its 63 outstanding loads = 16 KiB in flight, and every block costs a memory round trip per
+            // peer.  So the block is turned around in the wave's 16 KiB of LDS first (4-byte writes in accumulator layout,
+            // 16-byte reads along the rows: a lane then holds four consecutive columns of rows 2j + lane/32, j = 0..15), and a
+            // peer's values are 16 sixteen-byte loads per lane, issued eight at a time ("units") into a ring of six register
+            // buffers, five units (40 KiB per wave) in flight.  Every element sees the same additions in the same order as in
+            // accumulator layout.              static_assert(NW * 16384 <= POOL, "one 16 KiB staging area per wave");
+            constexpr int NBUF = 6;
+            unsigned char *st = smem + w * 16384;
+            __syncthreads();   // every wave has left the main loop's LDS reads behind
+            const uint32_t U = 2u * args.nPeers;   // units: peer u / 2, rows 16 (u & 1) .. of the block
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                if constexpr (RM)
+                    if (!(keptMb & (1u << mb))) continue;
+                const uint32_t lrow = lane >> 5, chunk = lane & 31;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t wrow = (r >> 2) * 8 + h * 4 + (r & 3);
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb) *(float *)(st + wrow * 512 + (((nb * 32 + c32) * 4) ^ (h << 7))) = getf(mb, nb, r);
+                }
+                v4f cur[16];
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const uint32_t wrow = j * 2 + lrow;
+                    cur[j] = *(const v4f *)(st + wrow * 512 + ((chunk * 16) ^ (((wrow >> 2) & 1) << 7)));
+                }
+                // peers and output go through buffer descriptors: a wave-uniform base per unit, one per-lane offset for all
+                // of them, and the row step as a scalar offset, so that a load costs no address arithmetic in vector registers
+                const int64_t rowInKept = (int64_t)(int32_t)out_row0 + (ws >> 1) * 32 * MB + mb * 32;
+                const uint32_t colW = ti.col + (ws & 1u) * 128;
+                const uint32_t pitchB = (uint32_t)args.peerLd * 4u;
+                const uint32_t voff = lrow * pitchB + chunk * 16u;
+                v4f buf[NBUF][8];
+                // (a unit past the last one is issued with an empty descriptor: its loads return zeros without touching memory,
+                // so every turn of the ring issues and counts the same number of loads whatever the number of peers)
+                auto issue = [&](v4f (&b)[8], uint32_t u) {
+                    const float *base = (const float *)args.peers[umin(u >> 1, (uint32_t)kMaxRanks - 1u)] +
+                                        (args.peerRowOffset + rowInKept + (int64_t)((u & 1u) * 16u)) * args.peerLd + colW;
+                    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, u < U ? 0x7ffffff0 : 0, 0x00020000);
+#pragma unroll
+                    for (int jj = 0; jj < 8; ++jj)
+                        b[jj] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (2 * jj) * pitchB, 2 /* nt */));
+                };
+                if (U > 0) {
+#pragma unroll
+                    for (int q = 0; q < NBUF - 1; ++q) issue(buf[q], q);
+                    for (uint32_t u = 0; u < U; u += NBUF) {
+#pragma unroll
+                        for (int q = 0; q < NBUF; ++q) {   // unit u + q sits in buffer q and adds to rows 16 (q & 1) ..
+                            __builtin_amdgcn_sched_barrier(0);
+                            issue(buf[(q + NBUF - 1) % NBUF], u + q + NBUF - 1);
+                            __builtin_amdgcn_sched_barrier(0);
+                            if (u + q < U) {
+#pragma unroll
+                                for (int jj = 0; jj < 8; ++jj) {
+                                    v4f &c = cur[(q & 1) * 8 + jj];
+                                    c.x = __fadd_rn(c.x, buf[q][jj].x);
+                                    c.y = __fadd_rn(c.y, buf[q][jj].y);
+                                    c.z = __fadd_rn(c.z, buf[q][jj].z);
+                                    c.w = __fadd_rn(c.w, buf[q][jj].w);
+                                }
+                            }
+                        }
+                    }
+                }
+                // 16-bit output: a lane's four columns are eight bytes, a wave instruction covers two 256-byte row segments
+                const uint32_t pitchD = (uint32_t)args.ldd * 2u;
+                const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(
+                    (void *)((unsigned char *)args.d + (rowInKept * args.ldd + colW) * 2), 0, 0x7ffffff0, 0x00020000);
+                const uint32_t voffD = lrow * pitchD + chunk * 8u;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    uint32_t q0, q1, q2, q3;
+                    if (args.outDtype == DT_BF16) {
+                        q0 = f32_to_bf16_bits(cur[j].x); q1 = f32_to_bf16_bits(cur[j].y); q2 = f32_to_bf16_bits(cur[j].z); q3 = f32_to_bf16_bits(cur[j].w);
+                    } else {
+                        q0 = f32_to_f16_bits(cur[j].x); q1 = f32_to_f16_bits(cur[j].y); q2 = f32_to_f16_bits(cur[j].z); q3 = f32_to_f16_bits(cur[j].w);
+                    }
+                    const v2i pk = {(int)((q0 & 0xffffu) | (q1 << 16)), (int)((q2 & 0xffffu) | (q3 << 16))};
+                    __builtin_amdgcn_raw_buffer_store_b64(pk, rd, voffD, (2 * j) * pitchD, 0);
+                }
+            }
+        } else {
         // one fp32 partial of the tile, added from global memory 32 rows (64 loads per lane) at a time
         // (RM: a block that is not kept adds the first 32 kept rows of the peer instead -- valid memory, and its sums are
         // never stored; skipping it would put control flow around the accumulators, which costs far more than the loads)
@@ -819,6 +925,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             const uint32_t wrow = j * 4 + (lane >> 4), chunk = lane & 15;
             const v4i v = *(const v4i *)(st + wrow * 256 + ((chunk * 16) ^ (((wrow >> 2) & 1) << 7)));
             *(v4i *)(dwave + (size_t)wrow * args.ldd * 2 + chunk * 16) = v;
+        }
         }
     } else if (args.flags & GF_OUTBOUND_STORE) {
         // fp32 tile of another rank, to the tile-linear workspace (rows wsRow .., n0 columns).  A lane holds single columns
@@ -941,10 +1048,10 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
 }
 
 // One workgroup per tile, or per k slice of a tile.
-template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false>
-__global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs args)
+template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false, int NS = 3, bool PP = false>
+__global__ void __launch_bounds__(128 * WM, NS == 3 ? 2 : 1) gemm_dma_kernel(const GemmArgs args)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<WM>::BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<WM, NS>::BYTES];
     // A launch with few tiles can cut every tile's k range into kSlices pieces, one workgroup each (128-row tiles
     // only): position `pos` of the launch order runs as kSlices workgroups that stay in the position's XCD column.
     uint32_t pos = blockIdx.x + args.taskBase, slice = 0;   // (taskBase is zero for k-sliced launches)
@@ -959,7 +1066,7 @@ __global__ void __launch_bounds__(128 * WM, 2) gemm_dma_kernel(const GemmArgs ar
             pos = blockIdx.x / kSlices;
         }
     }
-    dma_tile<DT, WM, TB, RM, RG, TA, 2>(args, smem, pos, slice, kSlices, 0);
+    dma_tile<DT, WM, TB, RM, RG, TA, 2, NS, PP>(args, smem, pos, slice, kSlices, 0);
 }
 
 // Reduce-scatter launches of a single round of workgroups (no more tiles than the 512 slots of the GPU): every kept 128-row
@@ -977,6 +1084,17 @@ __global__ void __launch_bounds__(256, 2) gemm_dma_split_kept_kernel(const GemmA
     else dma_tile<DT, 2, TB, false, false, false, 2>(args, smem, (j - keptPerXcd) * 8u + x, 0, 1, 0);
 }
 
+// A launch of at most one workgroup per CU has the whole LDS of a CU for each workgroup.  When its operands are too large to
+// come out of the L2s (48 MB of A and B or more: they stream from HBM or the Infinity Cache, whose latency the two steps of
+// look-ahead of the three-stage ring do not cover) it runs the six-stage ring with the pipelined peer loads.  Measured with
+// the variants alternating launch by launch, W8A8 with explicit kept rows at K = N = 8192: M = 256 / 512 / 1024 rows 108 /
+// 121 / 148 us on three stages, 54 / 67 / 91 with six, 42 / 60 / 92 with the pipelined peer loads as well.  Small operands do
+// not gain: config 2 (42 MB) 47.9 -> 49.6 us, config 1 18.2 -> 20.7 (and 23.6 with the pipelined peer loads).
+inline bool deep_ring(const GemmArgs &a, uint32_t workgroups, uint64_t es /* bytes per operand element */)
+{
+    return workgroups <= 256u && (uint64_t)a.K * es * ((uint64_t)a.M * (a.sched.op == OP_ALLGATHER ? a.sched.P : 1u) + a.N) >= (48ull << 20);
+}
+
 // Launch of the 128-row geometry: one instantiation per operand layout (A as [m][k] or [k][m], B as [k][n] or [n][k]) and
 // for ragged problems; one workgroup per tile, or per k slice of a tile.
 template <uint32_t DT>
@@ -987,6 +1105,8 @@ inline int launch_dma_128(const GemmArgs &args, hipStream_t s)
         case 0:
             if (const uint32_t keptPerXcd = split_kept_tiles(args, args.K * (DT == DT_I8 ? 1u : 2u) / 64u))
                 hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT, false>), dim3(args.sched.coreLoops + 8u * keptPerXcd), block, 0, s, args, keptPerXcd);
+            else if (deep_ring(args, grid.x, DT == DT_I8 ? 1u : 2u))
+                hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false, 6, true>), grid, block, 0, s, args);
             else
                 hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false>), grid, block, 0, s, args);
             break;

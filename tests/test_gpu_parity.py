@@ -1080,6 +1080,42 @@ def test_float_config3_full_size_properties():
         assert abs(csh[task] - want_cs) <= 1e-6 * 128 * 256, task
 
 
+@pytest.mark.parametrize("case", [(1024, 8192, 8192, 8, 3, None), (512, 8192, 8192, 4, 1, (0, 2)), (1024, 8192, 6144, 2, 0, None)])
+def test_quant_rs_operands_streamed_from_hbm(case):
+    """At most one workgroup per CU and 48 MB of operands or more: the launch runs the six-stage ring with the pipelined
+    row-layout peer loads (whole tiles kept; one case k-sliced through a workspace, one with a single peer).  Same bits as
+    every other route: int32 accumulators, kept int32 block and every output element equal the oracle's."""
+    M, N, K, P, rank, ks = case
+    r = quant_case(np.random.default_rng(90 + rank), M, N, K, P, rank, bias=True, launches=2, kslices=ks)
+    assert r["exact"] == r["total"]
+
+
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+def test_float_reduce_scatter_operands_streamed_from_hbm(dtype):
+    """The same route for 2-byte operands: 256 tiles, 72 MB of A and B, a row sample against the oracle and the whole local
+    partial through row sums against fp64."""
+    _need_gpu()
+    M, N, K, P, rank = 1024, 8192, 4096, 8, 6
+    g = torch.Generator(device=DEV).manual_seed(71)
+    td = TORCH_DT[dtype]
+    A = torch.randn((M, K), device=DEV, generator=g).to(td)
+    B = (torch.randn((K, N), device=DEV, generator=g) * 0.02).to(td)
+    rows = M // P
+    peers = [torch.randn((rows, N), device=DEV, generator=g) for _ in range(P - 1)]
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    out = ops.matmul_reduce_scatter(A, B, peers, rank, P, acc_dump=dump)
+    torch.cuda.synchronize()
+    want_rows = A.double() @ B.double().sum(1)
+    assert (dump.double().sum(1) - want_rows).abs().max().item() <= 5e-2
+    sel = np.arange(rank * rows, (rank + 1) * rows, 5)
+    part, want = oracle.matmul_reduce(host16(A[sel]), host16(B), dtype, 0, len(sel),
+                                      [p[sel - rank * rows].cpu().numpy() for p in peers], want_partial=True)
+    full = part + sum(p[sel - rank * rows].cpu().numpy() for p in peers)
+    _check_float(host16(out[sel - rank * rows]), want, full, dtype, K)
+    assert (ulp_diff16(host16(out[sel - rank * rows]), want) <= 1).mean() > 0.999
+    assert np.abs(dump[sel].cpu().numpy() - part).max() <= 2e-3
+
+
 @pytest.mark.parametrize("M", [1, 16, 64, 128, 512])
 def test_quant_config5_full_size(M):
     """W8A8 decode sweep config at full size (K = N = 8192, P = 8, rank 0 keeps rows [0, ceil(M/8))): kept rows bit
