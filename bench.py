@@ -11,6 +11,7 @@ in HBM before the timed region.  Prints ONE JSON line.
     python bench.py --mode decode   # BASELINE config 5: skinny-M sweep, K = N = 8192, GB/s per M (HBM-bound)
     python bench.py --mode float    # BASELINE configs 3 (fp16 reduce-scatter), 2 (bf16 all-gather) and 1 (fp16 all-reduce)
     python bench.py --mode ceiling  # what the int8 matrix pipes sustain on this box without any memory traffic (power-limited)
+    python bench.py --mode probes   # the peer-partial stream on its own; LDS and direct-to-LDS copy rates of a CU
     python bench.py --mode sweep    # dynamic_tiling's sweep protocol on the MI355X-side knobs; writes the reference's result.csv
 """
 import argparse
@@ -299,12 +300,74 @@ def mfma_ceiling(args, torch, L, dev):
         "ceiling": res}))
 
 
+def memory_probes(args, torch, L, dev):
+    """Two measurement helpers behind the design notes: (1) the peer-partial stream of config 4 on its own (128 workgroups pull
+    seven [1024,4096] fp32 partials, rotating over four sets so that they come from HBM), in the accumulator layout of the
+    kept epilogue and in row layout with 16-byte loads at several depths; (2) what a CU's LDS and its direct-to-LDS copy path
+    deliver (bytes per second and per clock at the clock the device reports)."""
+    import ctypes as C
+    so = L.load()
+    stream = lambda: torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device=dev).manual_seed(20250101)
+    rows, n, P, sets = 1024, 4096, 7, 4
+    bufs = [[torch.randn((rows, n), device=dev, generator=g) for _ in range(P)] for _ in range(sets)]
+    ptrs = [torch.tensor([b.data_ptr() for b in bs], dtype=torch.int64, device=dev) for bs in bufs]
+    sink = torch.zeros(512 * 256, dtype=torch.int32, device=dev)
+    nbytes = P * rows * n * 4
+
+    def timed(fn, reps):
+        for i in range(max(args.warmup, 2)):
+            fn(i)
+        ts = []
+        for i in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e-3)
+        return sum(ts) / len(ts), min(ts)
+
+    stream_res = []
+    for name, layout, depth in (("accumulator layout, 64 four-byte loads per batch", 0, 0), ("row layout, 16-byte loads, 2 units in flight", 1, 2),
+                                ("row layout, 3 units", 1, 3), ("row layout, 4 units", 1, 4), ("row layout, 6 units", 1, 6)):
+        def fn(i):
+            rc = so.catcoc_probe_peer_stream(stream(), layout, depth, ptrs[i % sets].data_ptr(), P, rows, n, sink.data_ptr())
+            assert rc == 0
+        mean, best = timed(fn, max(args.steps, 20))
+        stream_res.append({"variant": name, "us_mean": round(mean * 1e6, 1), "us_min": round(best * 1e6, 1),
+                           "TBps_mean": round(nbytes / mean / 1e12, 2), "TBps_at_min": round(nbytes / best / 1e12, 2)})
+    src = torch.randint(-127, 128, (32768,), dtype=torch.int8, device=dev, generator=g)
+    iters = 20000
+    cu, mhz = C.c_int(), C.c_int()
+    so.catcoc_device_info(C.byref(cu), C.byref(mhz), None, 0)
+    lds_res = []
+    for wgs in (256, 512):
+        for name, mode, rd, wr in (("16-byte LDS reads", 1, 8192, 0), ("transposing 8-byte LDS reads", 2, 8192, 0), ("both kinds of reads", 3, 16384, 0),
+                                   ("direct-to-LDS copies (source in the caches)", 4, 0, 6144), ("both reads and copies", 7, 16384, 6144)):
+            def fn(i):
+                rc = so.catcoc_probe_lds(stream(), mode, wgs, iters, src.data_ptr(), sink.data_ptr())
+                assert rc == 0
+            mean, best = timed(fn, 5)
+            per_cu = (rd + wr) * 4.0 * iters * (wgs / float(cu.value))
+            lds_res.append({"what": name, "workgroups_per_cu": wgs // 256, "ms_min": round(best * 1e3, 3), "GBps_per_cu": round(per_cu / best / 1e9, 1),
+                            "bytes_per_clock_per_cu_at_%d_MHz" % mhz.value: round(per_cu / best / (mhz.value * 1e6), 1),
+                            "read_share": round(rd / float(rd + wr), 2)})
+    head = stream_res[0]
+    print(json.dumps({
+        "metric": "peer-partial stream of config 4 on its own (7 x [1024,4096] fp32, 128 workgroups), accumulator layout", "value": head["TBps_mean"],
+        "unit": "TB/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": max(args.warmup, 2), "ms_per_step": head["us_mean"] / 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "measurement helpers: catcoc_probe_peer_stream and catcoc_probe_lds"},
+        "peer_stream": stream_res, "lds_and_copy_path": lds_res}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode", "float", "sweep", "ceiling"], default="kept",
+    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode", "float", "sweep", "ceiling", "probes"], default="kept",
                     help="kept: non-kept tiles are folded into checksums (BASELINE's literal outputs); "
                          "outbound: they are also stored as fp32 to the symmetric workspace")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -354,6 +417,9 @@ def main():
         return
     if args.mode == "sweep":
         tiling_sweep(args, torch, L, ops, dev)
+        return
+    if args.mode == "probes":
+        memory_probes(args, torch, L, dev)
         return
     if args.mode == "ceiling":
         mfma_ceiling(args, torch, L, dev)

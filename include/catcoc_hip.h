@@ -391,6 +391,20 @@ CATCOC_API uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t 
  * 512 * 4 * steps * 16 * 65536.  It measures what the matrix pipes sustain for that data on the box at hand (they are
  * power-limited); bench.py --mode ceiling reports it next to the operator's rate.  Returns 0 on success. */
 CATCOC_API int catcoc_probe_mfma_int8(void *stream, uint32_t ldsReads, uint32_t steps, const uint8_t *pattern, uint8_t *sink);
+/* Measurement helper (no counterpart in the reference): the peer-partial stream of a reduce-scatter launch on its own.  One
+ * workgroup per 128x256 tile of a [rows, n] fp32 block (row pitch n; rows % 128 == 0, n % 256 == 0) adds up the nPeers
+ * partials at peers[] (a DEVICE array of device pointers).  layout 0: accumulator layout, 64 four-byte loads per lane, peer
+ * and 32-row block, awaited before they are added (the kept epilogue of the 128-row kernel); layout 1: row layout, sixteen-byte
+ * loads in units of eight with `depth` (2, 3, 4 or 6) units in flight (the pipelined epilogue; nPeers must be 7).
+ * sink: tiles * 256 * 4 bytes.  Returns 0 on success. */
+CATCOC_API int catcoc_probe_peer_stream(void *stream, uint32_t layout, uint32_t depth, const void *const *peers, uint32_t nPeers,
+                                        uint32_t rows, uint32_t n, uint8_t *sink);
+/* Measurement helper (no counterpart in the reference): LDS read and direct-to-LDS copy rates of a CU.  `workgroups` (256 = one
+ * per CU, 512 = two) workgroups of four waves with 72 KiB of LDS run `iters` iterations; per iteration and wave, by mode bit:
+ * 1 = eight 16-byte LDS reads (8 KiB), 2 = sixteen transposing 8-byte LDS reads (8 KiB), 4 = six 1 KiB direct-to-LDS copies from
+ * the 24 KiB at `src` (device memory, 16-byte aligned; it stays in the caches).  Modes 1, 2, 3, 4, 7.  sink: workgroups * 256 * 4
+ * bytes.  Returns 0 on success. */
+CATCOC_API int catcoc_probe_lds(void *stream, uint32_t mode, uint32_t workgroups, uint32_t iters, const uint8_t *src, uint8_t *sink);
 
 /* Library / device information: fills cuCount, clockMHz of the current device; returns 0 on success. */
 CATCOC_API int catcoc_device_info(int *cuCount, int *clockMHz, char *name, int nameLen);
