@@ -304,8 +304,10 @@ def memory_probes(args, torch, L, dev):
     """Two measurement helpers behind the design notes: (1) the peer-partial stream of config 4 on its own (128 workgroups pull
     seven [1024,4096] fp32 partials, rotating over four sets so that they come from HBM), in the accumulator layout of the
     kept epilogue and in row layout with 16-byte loads at several depths; (2) what a CU's LDS and its direct-to-LDS copy path
-    deliver (bytes per second and per clock at the clock the device reports)."""
+    deliver (bytes per second and per clock at the clock the device reports); (3) how much a workgroup that streams from HBM
+    or L2 slows the tile copies of the other workgroup on its CU."""
     import ctypes as C
+    import numpy as np
     so = L.load()
     stream = lambda: torch.cuda.current_stream().cuda_stream
     g = torch.Generator(device=dev).manual_seed(20250101)
@@ -353,13 +355,32 @@ def memory_probes(args, torch, L, dev):
             lds_res.append({"what": name, "workgroups_per_cu": wgs // 256, "ms_min": round(best * 1e3, 3), "GBps_per_cu": round(per_cu / best / 1e9, 1),
                             "bytes_per_clock_per_cu_at_%d_MHz" % mhz.value: round(per_cu / best / (mhz.value * 1e6), 1),
                             "read_share": round(rd / float(rd + wr), 2)})
+    # (3) a streaming neighbour on the CU
+    hot = torch.randint(-127, 128, (256 * 98304 + 256 * 65536,), dtype=torch.int8, device=dev, generator=g)
+    big = torch.zeros(1 << 28, dtype=torch.float32, device=dev)
+    ticks = torch.zeros(256, dtype=torch.int64, device=dev)
+    hwid = torch.zeros(512, dtype=torch.int32, device=dev)
+    nsteps = 200
+    nb_res = []
+    for rep in range(2):
+        for mode, name in ((0, "the CU's other workgroup exits at once"), (1, "it streams from HBM (batches of 64 four-byte loads, awaited)"),
+                           (2, "it streams the same way from L2")):
+            rc = so.catcoc_probe_neighbour(stream(), mode, nsteps, hot.data_ptr(), big.data_ptr(), sink.data_ptr(), ticks.data_ptr(), hwid.data_ptr())
+            assert rc == 0
+            torch.cuda.synchronize()
+            t = ticks.cpu().numpy() / 100.0   # us
+            h = hwid.cpu().numpy()
+            if rep == 1:
+                nb_res.append({"neighbour": name, "us_per_copy_step_median": round(float(np.median(t)) / nsteps, 3),
+                               "us_per_copy_step_max": round(float(t.max()) / nsteps, 3),
+                               "pairs_w_and_w_plus_256_on_one_cu": int((h[:256] == h[256:]).sum())})
     head = stream_res[0]
     print(json.dumps({
         "metric": "peer-partial stream of config 4 on its own (7 x [1024,4096] fp32, 128 workgroups), accumulator layout", "value": head["TBps_mean"],
         "unit": "TB/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": max(args.warmup, 2), "ms_per_step": head["us_mean"] / 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "measurement helpers: catcoc_probe_peer_stream and catcoc_probe_lds"},
-        "peer_stream": stream_res, "lds_and_copy_path": lds_res}))
+        "peer_stream": stream_res, "lds_and_copy_path": lds_res, "streaming_neighbour": nb_res}))
 
 
 def main():

@@ -405,6 +405,15 @@ CATCOC_API int catcoc_probe_peer_stream(void *stream, uint32_t layout, uint32_t 
  * the 24 KiB at `src` (device memory, 16-byte aligned; it stays in the caches).  Modes 1, 2, 3, 4, 7.  sink: workgroups * 256 * 4
  * bytes.  Returns 0 on success. */
 CATCOC_API int catcoc_probe_lds(void *stream, uint32_t mode, uint32_t workgroups, uint32_t iters, const uint8_t *src, uint8_t *sink);
+/* Measurement helper (no counterpart in the reference): what a streaming workgroup costs the other workgroup on its CU.  512
+ * workgroups, two per CU (w and w + 256).  The first 256 run the copy side of a main loop -- per step six 1 KiB direct-to-LDS
+ * copies per wave, two steps ahead, from 96 KiB of their own inside `hot` (device memory, 256 * 98304 + 256 * 65536 bytes,
+ * 16-byte aligned) -- for `steps` steps and leave their duration in ticks[w] (100 MHz ticks).  The other 256 exit at once
+ * (mode 0), or fetch steps / 2 batches of 64 four-byte loads per lane, each batch awaited, from 4 MiB of their own inside `big`
+ * (1 GiB of device memory; mode 1) or from 64 KiB of their own at the end of `hot` (mode 2).  hwid[w], w < 512: bits 0-7 CU /
+ * shader array / shader engine of the workgroup, bits 8.. its XCD.  sink: 256 * 256 * 4 bytes.  Returns 0 on success. */
+CATCOC_API int catcoc_probe_neighbour(void *stream, uint32_t mode, uint32_t steps, const uint8_t *hot, const uint8_t *big, uint8_t *sink,
+                                      uint64_t *ticks, uint32_t *hwid);
 
 /* Library / device information: fills cuCount, clockMHz of the current device; returns 0 on success. */
 CATCOC_API int catcoc_device_info(int *cuCount, int *clockMHz, char *name, int nameLen);

@@ -203,6 +203,63 @@ __global__ void __launch_bounds__(256, 2) probe_lds_kernel(const unsigned char *
     sink[blockIdx.x * 256 + tid] = x;
 }
 
+// ---- a streaming neighbour on the CU ---------------------------------------------------------------------------------
+// 512 workgroups with 72 KiB of LDS each, two per CU (workgroups w and w + 256 land on one CU; their HW_ID words are
+// returned so that the caller can check).  The first 256 run the copy side of a main loop and time themselves: per step six
+// 1 KiB direct-to-LDS copies per wave from a per-workgroup region that stays in L2, two steps ahead, a barrier and a pause of
+// the length of a step's MFMAs.  The other 256 exit at once (mode 0) or, like a kept tile's epilogue, fetch batches of 64
+// four-byte loads per lane and await each batch, from 4 MiB of their own each (mode 1: HBM) or from 64 KiB each (mode 2: L2).
+__global__ void __launch_bounds__(256, 2) probe_neighbour_kernel(const unsigned char *hot, const float *big, uint32_t mode, uint32_t steps,
+                                                                 float *sink, unsigned long long *ticks, uint32_t *hwid)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[72 * 1024];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const uint32_t ws = __builtin_amdgcn_readfirstlane((uint32_t)(tid >> 6));
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(CATCOC_LDS unsigned char *)smem;
+    if (tid == 0) {
+        uint32_t hw, xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        hwid[blockIdx.x] = ((hw >> 8) & 0xffu) | (xcc << 8);   // CU, shader array, shader engine; XCD
+    }
+    if (blockIdx.x < 256) {
+        const unsigned char *g = hot + (size_t)blockIdx.x * 98304 + (ws * 6) * 1024 + lane * 16;
+        const unsigned long long t0 = wall_clock64();
+        auto issue = [&](uint32_t step) {
+            const unsigned char *p = g + (step & 3u) * 24576;
+#pragma unroll
+            for (int j = 0; j < 6; ++j) dma16_at(p + j * 1024, lds0 + (step % 3u) * 24576 + (ws * 6 + j) * 1024);
+        };
+        issue(0);
+        issue(1);
+        for (uint32_t it = 0; it < steps; ++it) {
+            CATCOC_WAIT_VMCNT(6);
+            barrier_keep_vmem();
+            issue(it + 2);
+            __builtin_amdgcn_s_sleep(7);   // about 500 cycles
+        }
+        CATCOC_WAIT_VMCNT(0);
+        const unsigned long long t1 = wall_clock64();
+        if (tid == 0) ticks[blockIdx.x] = t1 - t0;   // 100 MHz ticks
+    } else if (mode != 0) {
+        const uint32_t v = blockIdx.x - 256;
+        const float *src = mode == 1 ? big + (size_t)v * (1u << 20) : (const float *)(hot + 256 * 98304) + (size_t)v * 16384;
+        const uint32_t span = mode == 1 ? (1u << 20) : 16384u;   // floats
+        float acc = 0;
+        for (uint32_t b = 0; b < steps / 2; ++b) {
+            float pv[64];
+            const float *p = src + (b * 16384u + ws * 4096u + lane) % span;
+#pragma unroll
+            for (int r = 0; r < 64; ++r) pv[r] = __builtin_nontemporal_load(p + r * 64);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < 64; ++r) acc += pv[r];
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        sink[v * 256 + tid] = acc;
+    }
+}
+
 }  // namespace catcoc
 
 extern "C" int catcoc_probe_mfma_int8(void *stream, uint32_t ldsReads, uint32_t steps, const uint8_t *pattern, uint8_t *sink)
@@ -247,5 +304,14 @@ extern "C" int catcoc_probe_lds(void *stream, uint32_t mode, uint32_t workgroups
         case 7: hipLaunchKernelGGL(catcoc::probe_lds_kernel<7>, grid, block, 0, s, src, iters, (int *)sink); break;
         default: return 1;
     }
+    return (int)hipGetLastError();
+}
+
+extern "C" int catcoc_probe_neighbour(void *stream, uint32_t mode, uint32_t steps, const uint8_t *hot, const uint8_t *big, uint8_t *sink,
+                                      uint64_t *ticks, uint32_t *hwid)
+{
+    if (hot == nullptr || big == nullptr || sink == nullptr || ticks == nullptr || hwid == nullptr || mode > 2 || (uintptr_t)hot % 16 != 0) return 1;
+    hipLaunchKernelGGL(catcoc::probe_neighbour_kernel, dim3(512), dim3(256), 0, (hipStream_t)stream, hot, (const float *)big, mode, steps, (float *)sink,
+                       (unsigned long long *)ticks, hwid);
     return (int)hipGetLastError();
 }

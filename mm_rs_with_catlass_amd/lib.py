@@ -73,7 +73,7 @@ EXPORTS = [
     "catcoc_device_info", "catcoc_version",
     "catcoc_pipelined_quant_matmul_reduce_scatter", "catcoc_pipelined_matmul_reduce_scatter", "catcoc_reduce_add",
     "catcoc_verify", "catcoc_comm_block_idx_ex", "catcoc_comm_core_loop", "catcoc_task_tiles",
-    "catcoc_probe_mfma_int8", "catcoc_probe_peer_stream", "catcoc_probe_lds",
+    "catcoc_probe_mfma_int8", "catcoc_probe_peer_stream", "catcoc_probe_lds", "catcoc_probe_neighbour",
 ]
 
 _lib = None
@@ -192,6 +192,8 @@ def load():
     L.catcoc_probe_peer_stream.restype = C.c_int
     L.catcoc_probe_lds.argtypes = [vp, u32, u32, u32, vp, vp]
     L.catcoc_probe_lds.restype = C.c_int
+    L.catcoc_probe_neighbour.argtypes = [vp, u32, u32, vp, vp, vp, vp, vp]
+    L.catcoc_probe_neighbour.restype = C.c_int
     _lib = L
     return L
 
