@@ -331,14 +331,29 @@ def memory_probes(args, torch, L, dev):
         return sum(ts) / len(ts), min(ts)
 
     stream_res = []
-    for name, layout, depth in (("accumulator layout, 64 four-byte loads per batch", 0, 0), ("row layout, 16-byte loads, 2 units in flight", 1, 2),
-                                ("row layout, 3 units", 1, 3), ("row layout, 4 units", 1, 4), ("row layout, 6 units", 1, 6)):
-        def fn(i):
-            rc = so.catcoc_probe_peer_stream(stream(), layout, depth, ptrs[i % sets].data_ptr(), P, rows, n, sink.data_ptr())
-            assert rc == 0
-        mean, best = timed(fn, max(args.steps, 20))
-        stream_res.append({"variant": name, "us_mean": round(mean * 1e6, 1), "us_min": round(best * 1e6, 1),
-                           "TBps_mean": round(nbytes / mean / 1e12, 2), "TBps_at_min": round(nbytes / best / 1e12, 2)})
+    evict = torch.zeros(1 << 27, dtype=torch.float32, device=dev)   # 512 MiB written between launches: nothing stays in the caches
+    for wrows in (128, rows):   # 16 workgroups (one tile row: far below what HBM delivers) and all 128
+        for name, layout, depth in (("accumulator layout, 64 four-byte loads per batch", 0, 0), ("row layout, 16-byte loads, 2 units in flight", 1, 2),
+                                    ("row layout, 3 units", 1, 3), ("row layout, 4 units", 1, 4), ("row layout, 6 units", 1, 6)):
+            def fn(i):
+                evict.add_(1.0)
+                rc = so.catcoc_probe_peer_stream(stream(), layout, depth, ptrs[i % sets].data_ptr(), P, wrows, n, sink.data_ptr())
+                assert rc == 0
+            ts = []
+            for i in range(max(args.steps, 20) + 2):
+                evict.add_(1.0)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                rc = so.catcoc_probe_peer_stream(stream(), layout, depth, ptrs[i % sets].data_ptr(), P, wrows, n, sink.data_ptr())
+                e1.record()
+                torch.cuda.synchronize()
+                assert rc == 0
+                ts.append(e0.elapsed_time(e1) * 1e-3)
+            ts = ts[2:]
+            mean, best = sum(ts) / len(ts), min(ts)
+            wb = P * wrows * n * 4
+            stream_res.append({"workgroups": wrows // 128 * (n // 256), "variant": name, "us_mean": round(mean * 1e6, 1), "us_min": round(best * 1e6, 1),
+                               "TBps_mean": round(wb / mean / 1e12, 2), "GBps_per_workgroup_mean": round(wb / mean / 1e9 / (wrows // 128 * (n // 256)), 1)})
     src = torch.randint(-127, 128, (32768,), dtype=torch.int8, device=dev, generator=g)
     iters = 20000
     cu, mhz = C.c_int(), C.c_int()
@@ -374,7 +389,7 @@ def memory_probes(args, torch, L, dev):
                 nb_res.append({"neighbour": name, "us_per_copy_step_median": round(float(np.median(t)) / nsteps, 3),
                                "us_per_copy_step_max": round(float(t.max()) / nsteps, 3),
                                "pairs_w_and_w_plus_256_on_one_cu": int((h[:256] == h[256:]).sum())})
-    head = stream_res[0]
+    head = [r for r in stream_res if r["workgroups"] == 128][0]
     print(json.dumps({
         "metric": "peer-partial stream of config 4 on its own (7 x [1024,4096] fp32, 128 workgroups), accumulator layout", "value": head["TBps_mean"],
         "unit": "TB/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": max(args.warmup, 2), "ms_per_step": head["us_mean"] / 1e3,

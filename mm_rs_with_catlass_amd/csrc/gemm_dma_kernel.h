@@ -790,7 +790,8 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             // 16-byte reads along the rows: a lane then holds four consecutive columns of rows 2j + lane/32, j = 0..15), and a
             // peer's values are 16 sixteen-byte loads per lane, issued eight at a time ("units") into a ring of six register
             // buffers, five units (40 KiB per wave) in flight.  Every element sees the same additions in the same order as in
-            // accumulator layout.              static_assert(NW * 16384 <= POOL, "one 16 KiB staging area per wave");
+            // accumulator layout.
+            static_assert(NW * 16384 <= POOL, "one 16 KiB staging area per wave");
             constexpr int NBUF = 6;
             unsigned char *st = smem + w * 16384;
             __syncthreads();   // every wave has left the main loop's LDS reads behind
