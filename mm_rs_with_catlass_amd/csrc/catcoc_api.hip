@@ -297,10 +297,10 @@ struct SplitkPlan {
 // Explicit kept rows with at least this many rows of A run the 128x256 direct-to-LDS kernel (k-sliced through the same
 // workspace) when the shape has full tiles and the kept rows are whole 32-row blocks.  Such launches have at most one
 // workgroup per CU and run the kernel's six-stage ring with the pipelined peer loads.  Measured at K = N = 8192 with kept
-// rows = M / 8, the two routes alternating launch by launch: M = 1024 91 against 155 us, M = 512 60 (two k slices) against
-// 75 us, M = 256 43 (four k slices) against 51 us.  n0 = 256 (with m0 0 or 128) in the tiling asks for the large tile
-// explicitly, n0 = 128 for the split-K kernel.
-constexpr uint32_t kLargeTileRows = 256;
+// rows = M / 8, the two routes alternating launch by launch and B coming from HBM (six copies, another one every launch):
+// M = 1024 106 against 166 us, M = 512 69 (two k slices) against 77 us, M = 256 50 (four k slices) against 48 us.  n0 = 256
+// (with m0 0 or 128) in the tiling asks for the large tile explicitly, n0 = 128 for the split-K kernel.
+constexpr uint32_t kLargeTileRows = 512;
 
 int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uint32_t transA, uint32_t transB, SplitkPlan &sp)
 {
