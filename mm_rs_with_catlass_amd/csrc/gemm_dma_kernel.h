@@ -1088,10 +1088,9 @@ __global__ void __launch_bounds__(256, 2) gemm_dma_split_kept_kernel(const GemmA
 // A launch of at most one workgroup per CU has the whole LDS of a CU for each workgroup.  When its operands are too large to
 // come out of the L2s (48 MB of A and B or more: they stream from HBM or the Infinity Cache, whose latency the two steps of
 // look-ahead of the three-stage ring do not cover) it runs the six-stage ring with the pipelined peer loads.  Measured with
-// the variants alternating launch by launch, W8A8 with explicit kept rows at K = N = 8192 (one B, resident in the Infinity
-// Cache): M = 256 / 512 / 1024 rows 108 /
-// 121 / 148 us on three stages, 54 / 67 / 91 with six, 42 / 60 / 92 with the pipelined peer loads as well.  Small operands do
-// not gain: config 2 (42 MB) 47.9 -> 49.6 us, config 1 18.2 -> 20.7 (and 23.6 with the pipelined peer loads).
+// the variants alternating launch by launch, W8A8 with explicit kept rows at K = N = 8192, B from HBM on every launch (six
+// copies): M = 512 140 us on three stages, 75 with six, 70 with the pipelined peer loads as well; M = 1024 158 / 102 / 106.
+// Small operands do not gain: config 2 (42 MB) 47.9 -> 49.6 us, config 1 18.2 -> 20.7 (and 23.6 with the pipelined peer loads).
 inline bool deep_ring(const GemmArgs &a, uint32_t workgroups, uint64_t es /* bytes per operand element */)
 {
     return workgroups <= 256u && (uint64_t)a.K * es * ((uint64_t)a.M * (a.sched.op == OP_ALLGATHER ? a.sched.P : 1u) + a.N) >= (48ull << 20);
