@@ -558,7 +558,10 @@ def main():
         c_acc = torch.empty((rows, N), dtype=torch.int32, device=dev)
         p_out = torch.empty((rows, N), dtype=torch.bfloat16, device=dev)
         comm = torch.cuda.Stream()
-        ptil = ops.default_tiling(M, K, N, P, m0=128, n0=256, k0=256)
+        # commInterval 4 is the smallest of the reference's own search space (tiling.h:19-22); with 256 workgroups as blockNum a
+        # comm round then holds all 1024 tasks (one GEMM round, one comm round).  Measured: commInterval 1 (four rounds) 255 us,
+        # 2 (two rounds) 191 us, 4 and more (one round) 151 us per call.
+        ptil = ops.default_tiling(M, K, N, P, m0=128, n0=256, k0=256, commInterval=4)
         p_ws = torch.empty(so.catcoc_get_workspace_size(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, C.byref(ptil), C.byref(desc0)) // 4,
                            dtype=torch.int32, device=dev)
 
@@ -575,6 +578,7 @@ def main():
         torch.cuda.synchronize()   # (both streams: the call's last event joins the comm stream back into the current one)
         p_s = (time.perf_counter() - t0) / n_p
         pipelined = {"ms_per_step": round(p_s * 1e3, 5), "TOPS": round(2.0 * M * N * K / p_s / 1e12, 2), "commInterval": int(ptil.commInterval),
+                     "rounds": int(-(-ntasks // (256 * int(ptil.commInterval)))),
                      "note": "catcoc_pipelined_quant_matmul_reduce_scatter: GEMM rounds and comm rounds on two streams, int32 "
                              "peers reduced before the dequant; wall time per call over %d calls" % n_p}
 
