@@ -169,7 +169,8 @@ def float_configs(args, torch, L, ops, dev):
     peers = [torch.randn((rows, N), device=dev, generator=g) for _ in range(P - 1)]
     cs = torch.zeros(4096, dtype=torch.float64, device=dev)
     out = torch.empty((rows, N), dtype=torch.float16, device=dev)
-    wall, kern = timed(lambda: ops.matmul_reduce_scatter(A, B, peers, rank, P, checksum=cs, out=out))
+    ws3 = torch.zeros(65536, dtype=torch.uint8, device=dev)   # counter block: the checksum halves of tiles that run as two workgroups meet here
+    wall, kern = timed(lambda: ops.matmul_reduce_scatter(A, B, peers, rank, P, checksum=cs, out=out, workspace=ws3))
     sel = np.arange(0, rows, 61)
     _, want = oracle.matmul_reduce(A[sel].view(torch.int16).cpu().numpy().view(np.uint16), B.view(torch.int16).cpu().numpy().view(np.uint16),
                                    oracle.FP16, 0, len(sel), [p[sel].cpu().numpy() for p in peers])

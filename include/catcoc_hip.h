@@ -103,6 +103,11 @@ typedef void (*CatcocKernelFuncPtr)(void *stream, uint64_t fftsAddr, uint8_t *a,
  * tiles, A as [m,k], XCD-aware order): tuning knobs like the tiling's, results are bit-identical either way. */
 #define CATCOC_FLAG_KEPT_WHOLE 0x10u
 #define CATCOC_FLAG_KEPT_SPLIT 0x20u
+/* A launch with split kept tiles has more workgroups than the GPU has slots for; the tiles that wait for a slot (they get the
+ * ones the kept halves leave) run as two 64-row workgroups as well, unless this flag is set.  With checksums (the default
+ * outbound mode) the two halves of such a task meet through the counter block of desc.workspace: without a workspace of at
+ * least CATCOC_WORKSPACE_COUNTER_BYTES (zeroed once, shared like any other) they stay whole.  Results are bit-identical. */
+#define CATCOC_FLAG_TAIL_WHOLE 0x40u
 
 /* Replaces the reference's `symmetricPtr` workspace + shmem_my_pe()/shmem_n_pes()
  * (examples/dynamic_tiling/impl/kernel/matmul_reduce_scatter.h:155-156): which
@@ -374,6 +379,12 @@ CATCOC_API uint32_t catcoc_launch_task(int commType, const CocTilingParams *tili
  * 0 = none: the launch then has one workgroup per task, else that many workgroups more).  For tools that size or
  * reason about the grid.  No counterpart in the reference. */
 CATCOC_API uint32_t catcoc_kept_split_tiles(int commType, int dataType, const CocTilingParams *tiling,
+                                            const CatcocSymmetricDesc *desc, uint32_t transA, uint32_t transB);
+/* How many tiles at the end of the launch order such a launch also runs as two 64-row workgroups each (see
+ * CATCOC_FLAG_TAIL_WHOLE): the tiles by which tasks + kept halves exceed the 512 workgroup slots of the GPU; 0 when the
+ * launch asks for checksums and desc carries no workspace.  The checksum buffer itself does not enter: pass the descriptor
+ * the launch will use (desc.checksum non-NULL or not).  No counterpart in the reference. */
+CATCOC_API uint32_t catcoc_tail_split_tiles(int commType, int dataType, const CocTilingParams *tiling,
                                             const CatcocSymmetricDesc *desc, uint32_t transA, uint32_t transB);
 /* The same with the tile: what workgroup `wg` of the launch computes, exactly as the kernel works it out (the
  * large-tile kernels take a division-free route through constants prepared per launch; this entry point is how

@@ -249,6 +249,10 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
             }
         }
     }
+    // a workspace also lets the checksum halves of tiles that run as two workgroups meet (its counter block)
+    if (a.skCount == nullptr && d->workspace != nullptr && (uintptr_t)d->workspace % 256 == 0 && d->workspaceBytes >= kCounterBlockBytes)
+        a.skCount = (uint32_t *)d->workspace;
+    if (d->flags & CATCOC_FLAG_TAIL_WHOLE) a.flags |= GF_TAIL_WHOLE;
     return 0;
 }
 
@@ -926,6 +930,20 @@ uint32_t catcoc_kept_split_tiles(int commType, int dataType, const CocTilingPara
     ok();
     if (!p.dma || p.args.sched.m0 != 128) return 0;
     return 8u * split_kept_tiles(p.args, p.args.K * elem_size(p.dtype) / 64u);
+}
+
+uint32_t catcoc_tail_split_tiles(int commType, int dataType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
+                                 uint32_t transA, uint32_t transB)
+{
+    Plan p;
+    CatcocSymmetricDesc d;
+    if (desc == nullptr || tiling == nullptr) { fail(E_NULL, "tiling and desc must be non-NULL"); return 0; }
+    d = *desc;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!d.peers[i]) d.peers[i] = (const void *)16;
+    if (make_plan(commType, dataType, tiling, &d, transA, transB, p)) return 0;
+    ok();
+    if (!p.dma || p.args.sched.m0 != 128) return 0;
+    return 8u * split_tail_tiles(p.args, split_kept_tiles(p.args, p.args.K * elem_size(p.dtype) / 64u));
 }
 
 uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags)

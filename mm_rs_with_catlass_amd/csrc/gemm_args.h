@@ -20,6 +20,7 @@ enum : uint32_t {
                                   // block, index (row / 128) * (N / 128) + col / 128
     GF_KEPT_WHOLE = 1u << 5,      // never run kept tiles as two 64-row workgroups
     GF_KEPT_SPLIT = 1u << 6,      // do so whenever the launch allows it (default: by tile count and k length)
+    GF_TAIL_WHOLE = 1u << 7,      // never run the tiles that wait for the slots of kept halves as two 64-row workgroups
     GF_RAGGED = 1u << 4,          // the last tile row of a rank and / or the last tile column are not full: such tiles are computed as
                                   // whole tiles moved up / left so that they end at the edge (they overlap their neighbours, whose
                                   // values they reproduce bit for bit); sums and workspace stores leave the overlap out
@@ -72,6 +73,21 @@ inline uint32_t split_kept_tiles(const GemmArgs &a, uint32_t kSteps)
     if (a.flags & GF_KEPT_WHOLE) return 0;
     if (!(a.flags & GF_KEPT_SPLIT) && !(s.coreLoops < 256u || (s.coreLoops <= 512u && kSteps <= 64u))) return 0;
     return xcd_uniform_kept(s, a.keptRank);
+}
+
+// Tiles per XCD at the END of the launch order that a launch with split kept tiles also runs as two 64-row workgroups: the
+// tiles by which the launch exceeds the 512 workgroup slots of the GPU (each of them inherits the slot of a kept half).
+// Their checksum halves meet through the counter block of a workspace: without one (and with checksums asked for) they
+// stay whole.
+inline uint32_t split_tail_tiles(const GemmArgs &a, uint32_t keptPerXcd)
+{
+    const SchedParams &s = a.sched;
+    if (keptPerXcd == 0 || (a.flags & GF_TAIL_WHOLE)) return 0;
+    if (!(a.flags & GF_OUTBOUND_STORE) && a.checksum != nullptr && (a.skCount == nullptr || s.coreLoops > 8192u)) return 0;
+    const uint32_t wgs = s.coreLoops + 8u * keptPerXcd;
+    if (wgs <= 512u) return 0;
+    const uint32_t over = (wgs - 512u) >> 3;
+    return over <= keptPerXcd && over + keptPerXcd <= (s.coreLoops >> 3) ? over : 0;
 }
 
 }  // namespace catcoc

@@ -135,6 +135,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     if constexpr (MB == 1) {
         ti.row += subRow;
         ti.rowInRank += subRow;
+        ti.wsRow += subRow;
     }
     uint32_t shiftM = 0, shiftN = 0;   // RG: rows / columns at the start of the tile that belong to the neighbouring tile
     if constexpr (RG) {
@@ -1042,7 +1043,31 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             Sum t = 0;
 #pragma unroll
             for (int i = 0; i < NW; ++i) t += red[i];
-            ((Sum *)args.checksum)[task] = t;
+            if constexpr (MB == 1) {
+                // The two 64-row halves of a task meet through a 64-bit word per task (the workspace's counter block, all zero
+                // between launches): each exchanges its sum, encoded so that it is never zero, into the word; the half that
+                // finds the other's sum there adds the two (either order gives the same bits), writes the task's checksum
+                // and clears the word.
+                unsigned long long enc;
+                if constexpr (DT == DT_I8) {
+                    enc = (unsigned long long)(t + (1ll << 62));   // |t| < 2^47
+                } else {
+                    enc = __builtin_bit_cast(unsigned long long, t);
+                    if (t != t) enc = 0x7ff8000000000000ull;
+                    enc += 1ull;
+                }
+                unsigned long long *word = (unsigned long long *)args.skCount + task;
+                const unsigned long long other = __hip_atomic_exchange(word, enc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (other != 0ull) {
+                    Sum o;
+                    if constexpr (DT == DT_I8) o = (long long)other - (1ll << 62);
+                    else o = __builtin_bit_cast(double, other - 1ull);
+                    ((Sum *)args.checksum)[task] = t + o;
+                    __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            } else {
+                ((Sum *)args.checksum)[task] = t;
+            }
         }
     }
 
@@ -1070,19 +1095,36 @@ __global__ void __launch_bounds__(128 * WM, NS == 3 ? 2 : 1) gemm_dma_kernel(con
     dma_tile<DT, WM, TB, RM, RG, TA, 2, NS, PP>(args, smem, pos, slice, kSlices, 0);
 }
 
-// Reduce-scatter launches of a single round of workgroups (no more tiles than the 512 slots of the GPU): every kept 128-row
-// tile runs as two 64-row workgroups.  A kept tile is the longest chain of such a launch (its main loop, then the peers'
-// partials from HBM) and nothing follows it, so the launch lasts as long as that chain; cut in two, each half streams half
-// the peers.  Launch order inside an XCD (workgroup id = 8 * j + xcd): j < 2 * kept tiles of the XCD -> kept tile j / 2, rows
-// 64 * (j & 1) ..; later j -> the other tiles in their usual order.  Requires the XCD-block order, the same number of kept
-// tiles on every XCD (keptPerXcd), whole tiles, A as [m,k], one launch for all tasks.
+// Reduce-scatter launches of a single round of workgroups (no more tiles than the 512 slots of the GPU) run some tiles as two
+// 64-row workgroups.  Positions of an XCD in launch order (workgroup id = 8 * j + xcd):
+//   the first keptPerXcd positions, the kept tiles: a kept tile is the longest chain of such a launch (its main loop, then the
+//     peers' partials from HBM) and nothing follows it, so the launch lasts as long as that chain; cut in two, each half
+//     streams half the peers, on two CUs;
+//   the last tailPerXcd positions: the kept halves make the launch larger than the workgroup slots of the GPU, and the tiles
+//     that have to wait for a slot get the ones the kept halves leave, about one tile time before the end; as halves they
+//     fill those slots for half a tile time (their checksum halves meet through the workspace's counter block).
+// Requires the XCD-block order, whole tiles, A as [m,k], one launch for all tasks.
 template <uint32_t DT, bool TB>
-__global__ void __launch_bounds__(256, 2) gemm_dma_split_kept_kernel(const GemmArgs args, const uint32_t keptPerXcd)
+__global__ void __launch_bounds__(256, 2) gemm_dma_split_kept_kernel(const GemmArgs args, const uint32_t keptPerXcd, const uint32_t tailPerXcd)
 {
     __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<2>::BYTES];
-    const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
-    if (j < 2u * keptPerXcd) dma_tile<DT, 2, TB, false, false, false, 1>(args, smem, (j >> 1) * 8u + x, 0, 1, (j & 1u) * 64u);
-    else dma_tile<DT, 2, TB, false, false, false, 2>(args, smem, (j - keptPerXcd) * 8u + x, 0, 1, 0);
+    const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3, n = args.sched.coreLoops >> 3;
+    const uint32_t whole = n - keptPerXcd - tailPerXcd;   // positions keptPerXcd .. keptPerXcd + whole - 1 run whole
+    uint32_t posJ, sub = 0;
+    bool half = true;
+    if (j < 2u * keptPerXcd) {
+        posJ = j >> 1;
+        sub = (j & 1u) * 64u;
+    } else if (j < 2u * keptPerXcd + whole) {
+        posJ = j - keptPerXcd;
+        half = false;
+    } else {
+        const uint32_t t = j - (2u * keptPerXcd + whole);
+        posJ = keptPerXcd + whole + (t >> 1);
+        sub = (t & 1u) * 64u;
+    }
+    if (half) dma_tile<DT, 2, TB, false, false, false, 1>(args, smem, posJ * 8u + x, 0, 1, sub);
+    else dma_tile<DT, 2, TB, false, false, false, 2>(args, smem, posJ * 8u + x, 0, 1, 0);
 }
 
 // A launch of at most one workgroup per CU has the whole LDS of a CU for each workgroup.  When its operands are too large to
@@ -1105,7 +1147,11 @@ inline int launch_dma_128(const GemmArgs &args, hipStream_t s)
     switch ((args.transA ? 4 : 0) | (args.transB ? 2 : 0) | ((args.flags & GF_RAGGED) ? 1 : 0)) {
         case 0:
             if (const uint32_t keptPerXcd = split_kept_tiles(args, args.K * (DT == DT_I8 ? 1u : 2u) / 64u))
-                hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT, false>), dim3(args.sched.coreLoops + 8u * keptPerXcd), block, 0, s, args, keptPerXcd);
+{
+                const uint32_t tailPerXcd = split_tail_tiles(args, keptPerXcd);
+                hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT, false>), dim3(args.sched.coreLoops + 8u * (keptPerXcd + tailPerXcd)), block, 0, s, args,
+                                   keptPerXcd, tailPerXcd);
+            }
             else if (deep_ring(args, grid.x, DT == DT_I8 ? 1u : 2u))
                 hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false, 6, true>), grid, block, 0, s, args);
             else
@@ -1114,7 +1160,11 @@ inline int launch_dma_128(const GemmArgs &args, hipStream_t s)
         case 1: hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, true, false>), grid, block, 0, s, args); break;
         case 2:
             if (const uint32_t keptPerXcd = split_kept_tiles(args, args.K * (DT == DT_I8 ? 1u : 2u) / 64u))
-                hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT, true>), dim3(args.sched.coreLoops + 8u * keptPerXcd), block, 0, s, args, keptPerXcd);
+{
+                const uint32_t tailPerXcd = split_tail_tiles(args, keptPerXcd);
+                hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT, true>), dim3(args.sched.coreLoops + 8u * (keptPerXcd + tailPerXcd)), block, 0, s, args,
+                                   keptPerXcd, tailPerXcd);
+            }
             else
                 hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, true, false, false, false>), grid, block, 0, s, args);
             break;

@@ -24,6 +24,7 @@ FLAG_REDUCE_INT32 = 4
 FLAG_LINEAR_ORDER = 8
 FLAG_KEPT_WHOLE = 0x10
 FLAG_KEPT_SPLIT = 0x20
+FLAG_TAIL_WHOLE = 0x40
 
 
 class CatcocError(RuntimeError):
@@ -69,7 +70,7 @@ EXPORTS = [
     "catcoc_get_task_count", "catcoc_get_tilings", "catcoc_check_comm_interval_reduce_scatter",
     "catcoc_check_comm_interval_allreduce", "catcoc_check_comm_interval_allgather", "catcoc_get_splitk_factor",
     "catcoc_default_tiling", "catcoc_swizzle_block_coord", "catcoc_splitk_block_coord", "catcoc_splitk_actual_k", "catcoc_splitk_launch_task",
-    "catcoc_allgather_block_coord", "catcoc_comm_block_idx", "catcoc_task_tile", "catcoc_workgroup_task", "catcoc_launch_task", "catcoc_launch_tile", "catcoc_kept_split_tiles",
+    "catcoc_allgather_block_coord", "catcoc_comm_block_idx", "catcoc_task_tile", "catcoc_workgroup_task", "catcoc_launch_task", "catcoc_launch_tile", "catcoc_kept_split_tiles", "catcoc_tail_split_tiles",
     "catcoc_device_info", "catcoc_version",
     "catcoc_pipelined_quant_matmul_reduce_scatter", "catcoc_pipelined_matmul_reduce_scatter", "catcoc_reduce_add",
     "catcoc_verify", "catcoc_comm_block_idx_ex", "catcoc_comm_core_loop", "catcoc_task_tiles",
@@ -142,6 +143,8 @@ def load():
     L.catcoc_launch_task.restype = u32
     L.catcoc_kept_split_tiles.argtypes = [C.c_int, C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32, u32]
     L.catcoc_kept_split_tiles.restype = u32
+    L.catcoc_tail_split_tiles.argtypes = [C.c_int, C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32, u32]
+    L.catcoc_tail_split_tiles.restype = u32
     L.catcoc_get_task_count.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc)]
     L.catcoc_get_task_count.restype = u32
     L.catcoc_get_tilings.argtypes = [C.POINTER(CocTilingParams), C.c_int, C.c_int, C.c_int, C.POINTER(CocTilingParams), C.c_int]

@@ -89,7 +89,10 @@ def _task_count(comm_type, t, d):
 
 
 def _kept_flag(kept_split):
-    """kept_split: None = the library decides, False = kept tiles whole, True = two 64-row workgroups where allowed."""
+    """kept_split: None = the library decides, False = kept tiles whole, True = two 64-row workgroups where allowed,
+    "kept-only" = as None but the tiles that wait for the kept halves' slots stay whole (CATCOC_FLAG_TAIL_WHOLE)."""
+    if kept_split == "kept-only":
+        return _l.FLAG_TAIL_WHOLE
     return 0 if kept_split is None else (_l.FLAG_KEPT_SPLIT if kept_split else _l.FLAG_KEPT_WHOLE)
 
 

@@ -560,6 +560,29 @@ def test_kept_split_choice_by_tile_count_and_k_length():
     assert split(Q, L.INT8, 1024, 7168, 4096, 8) == 16                # 128 tiles: fewer than CUs, any k
     assert split(RS, L.FP16, 4096, 1792, 4096, 8) == 64               # config 3: 512 tiles, 56 k steps
     assert split(RS, L.FP16, 4096, 2112, 4096, 8) == 0                # 66 k steps
+
+    # the tiles by which tasks + kept halves exceed the 512 workgroup slots run as halves too (catcoc_tail_split_tiles); their
+    # checksum halves need the counter block of a workspace
+    def tail(comm, dt, m, k, n, p, flags=0, checksum=False, workspace=False):
+        t = ops.default_tiling(m, k, n, p, m0=0, n0=0, k0=0)
+        d = L.make_desc(0, p, [16] * (p - 1))
+        d.flags = flags
+        if checksum:
+            d.checksum = 4096
+        if workspace:
+            d.workspace, d.workspaceBytes = 4096, 65536
+        r = so.catcoc_tail_split_tiles(comm, dt, C.byref(t), C.byref(d), 0, 0)
+        L.check()
+        return r
+    assert tail(Q, L.INT8, 4096, 1792, 4096, 8) == 64                               # 512 + 64 - 512
+    assert tail(Q, L.INT8, 4096, 1792, 4096, 8, checksum=True) == 0                 # no workspace for the checksum halves
+    assert tail(Q, L.INT8, 4096, 1792, 4096, 8, checksum=True, workspace=True) == 64
+    assert tail(Q, L.INT8, 4096, 1792, 4096, 8, L.FLAG_TAIL_WHOLE) == 0
+    assert tail(Q, L.INT8, 4096, 1792, 4096, 8, L.FLAG_KEPT_WHOLE) == 0
+    assert tail(Q, L.INT8, 3072, 1792, 4096, 8) == 0                                # 384 + 48 workgroups fit
+    assert tail(Q, L.INT8, 4096, 1792, 3584, 8) == 0                                # 448 + 56 workgroups fit
+    assert tail(Q, L.INT8, 8192, 1792, 4096, 8) == 0                                # no split kept tiles, no tail
+    assert tail(RS, L.FP16, 4096, 1792, 4096, 8, checksum=True, workspace=True) == 64
     assert split(RS, L.FP16, 8 * 296, 512, 1344, 8) == 0              # ragged problems keep whole tiles
     assert split(L.MATMUL_ALLREDUCE, L.FP16, 1024, 512, 1024, 2) == 0 # no kept-rank block to split
     assert split(Q, L.INT8, 4096, 1792, 4096, 1) == 0                 # no peers to stream

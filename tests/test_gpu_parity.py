@@ -215,6 +215,60 @@ def test_quant_rs_kept_tiles_whole_or_split_give_the_same_bits(tb):
         assert int(res[0][1].ne(0).sum()) >= ntasks * 7 // 8 - 2
 
 
+@pytest.mark.parametrize("kind", ["int8", "fp16"])
+def test_rs_tiles_that_wait_for_kept_halves_run_as_halves(kind):
+    """512 tiles with split kept tiles are 576 workgroups on 512 slots; with a workspace (the checksum halves of a task meet
+    through its counter block) the 64 tiles that wait run as two 64-row workgroups.  Outputs and per-task checksums equal those
+    of the launch with whole tiles bit for bit, the counter block is clean again, and without a workspace the launch falls back."""
+    _need_gpu()
+    import ctypes as C
+    M, N, K, P, rank = 4096, 4096, 320, 8, 5
+    g = torch.Generator(device=DEV).manual_seed(77)
+    rows = M // P
+    peers = [torch.randn((rows, N), device=DEV, generator=g) for _ in range(P - 1)]
+    if kind == "int8":
+        x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
+        x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=DEV, generator=g)
+        s1 = torch.empty(M, device=DEV).uniform_(0.005, 0.02, generator=g)
+        s2 = torch.empty(N, device=DEV).uniform_(0.001, 0.01, generator=g)
+        comm, dt, csdt = L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, torch.int64
+        run = lambda **kw: ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, rank, P, **kw)
+    else:
+        A = torch.randn((M, K), device=DEV, generator=g).half()
+        B = (torch.randn((K, N), device=DEV, generator=g) * 0.02).half()
+        comm, dt, csdt = L.MATMUL_REDUCE_SCATTER, L.FP16, torch.float64
+        run = lambda **kw: ops.matmul_reduce_scatter(A, B, peers, rank, P, **kw)
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    d.checksum, d.workspace, d.workspaceBytes = 4096, 4096, 65536
+    so = L.load()
+    assert so.catcoc_kept_split_tiles(comm, dt, C.byref(t), C.byref(d), 0, 0) == 64
+    assert so.catcoc_tail_split_tiles(comm, dt, C.byref(t), C.byref(d), 0, 0) == 64
+    res = {}
+    for name, kw in (("whole", dict(kept_split=False)), ("kept halves", dict(kept_split="kept-only")), ("kept and waiting halves", dict()),
+                     ("no workspace", dict(workspace=None))):
+        cs = torch.full((512,), -1, dtype=csdt, device=DEV)
+        ws = torch.zeros(65536, dtype=torch.uint8, device=DEV)
+        kw.setdefault("workspace", ws)
+        for _ in range(2):   # (the second launch finds the counter block as the first left it)
+            out = run(checksum=cs, **kw)
+        torch.cuda.synchronize()
+        assert not ws.any(), name
+        res[name] = (host16(out), cs.cpu().numpy())
+    for name in res:
+        assert np.array_equal(res[name][0], res["whole"][0]), name
+        assert np.array_equal(res[name][1], res["whole"][1]), name
+    # and the outbound mode: halves store their own rows of the workspace tile
+    need = so.catcoc_get_workspace_size(comm, dt, C.byref(t), C.byref(d))
+    obs = []
+    for kw in (dict(kept_split=False), dict()):
+        ob = torch.zeros(need // 4, dtype=torch.float32, device=DEV)
+        run(outbound=ob, **kw)
+        torch.cuda.synchronize()
+        obs.append(ob.cpu().numpy())
+    assert np.array_equal(obs[0].view(np.uint32), obs[1].view(np.uint32))
+
+
 @pytest.mark.parametrize("shape", [(32, 129, 100), (24, 7, 3), (4 * 23, 45, 68), (4, 128, 512)])
 def test_quant_rs_general_shapes(shape):
     # K not a multiple of 16 or N not a multiple of 4: the general kernel (incl. the reference's own
