@@ -97,7 +97,7 @@ typedef void (*CatcocKernelFuncPtr)(void *stream, uint64_t fftsAddr, uint8_t *a,
 #define CATCOC_FLAG_REDUCE_INT32 0x4u
 /* Keep the linear workgroup -> task order (no XCD-aware chunking). */
 #define CATCOC_FLAG_LINEAR_ORDER 0x8u
-/* Reduce-scatter launches of one round of workgroups (at most 512 tiles of 128x256 with at most 64 k steps of 64 bytes,
+/* Reduce-scatter launches of one round of workgroups (at most 512 tiles of 128x256 with at most 80 k steps of 64 bytes,
  * or fewer than 256 tiles) run every kept tile as two 64-row workgroups, which halves the chain of peer partials a
  * workgroup adds; the library decides by those two numbers.  KEPT_WHOLE never splits, KEPT_SPLIT splits whenever the launch allows it (whole
  * tiles, A as [m,k], XCD-aware order): tuning knobs like the tiling's, results are bit-identical either way. */

@@ -60,10 +60,12 @@ inline uint32_t launch_positions(const GemmArgs &a) { return a.taskCount ? a.tas
 
 // Kept tiles per XCD when a launch qualifies for gemm_dma_split_kept_kernel, else 0: a whole reduce-scatter launch in the
 // XCD-block order, A as [m,k], the kept rows exactly the kept rank's block with peers to stream, and by default either
-// fewer tiles than CUs or at most one round of workgroups (512 tiles) with at most 64 k steps per tile.  Measured with
-// the two variants alternating launch by launch (W8A8, N = 4096, whole -> split, us): 512 tiles with 28 / 40 / 56 / 72 /
-// 80 / 112 k steps 54.4 -> 40.5 / 65.7 -> 54.5 / 79.6 -> 73.7 / 92.3 -> 91.8 / 102.9 -> 106.2 / 128.7 -> 140.9; 128 tiles
-// with 112 steps 67.3 -> 49.8; 768 tiles 59.3 -> 59.1; 1024 tiles 74.8 -> 83.3.  GF_KEPT_WHOLE / GF_KEPT_SPLIT override.
+// fewer tiles than CUs or at most one round of workgroups (512 tiles) with at most 80 k steps per tile.  Measured with
+// the two variants alternating launch by launch and the inputs rotating over several sets (W8A8, N = 4096, 512 tiles, whole ->
+// split with the waiting tiles as halves, us): 28 / 56 / 64 / 72 / 80 / 112 k steps 55.6 -> 42.7 / 77.4 -> 70.7 / 87.1 -> 84.4 /
+// 90.4 -> 86.9 / 97.6 -> 95.9 / 125.8 -> 130.7; fp16 56 / 64 / 80 / 112 steps 78.5 -> 72.8 / 87.9 -> 84.8 / 98.1 -> 97.5 / 126.9 ->
+// 131.8; 128 tiles with 112 steps 67.3 -> 49.8; 768 tiles 59.3 -> 59.1; 1024 tiles 74.8 -> 83.3.  GF_KEPT_WHOLE / GF_KEPT_SPLIT
+// override.
 inline uint32_t split_kept_tiles(const GemmArgs &a, uint32_t kSteps)
 {
     const SchedParams &s = a.sched;
@@ -71,7 +73,7 @@ inline uint32_t split_kept_tiles(const GemmArgs &a, uint32_t kSteps)
         a.transA || a.nPeers == 0 || a.keptBegin != a.keptRank * s.mRank || a.keptRows != s.mRank)
         return 0;
     if (a.flags & GF_KEPT_WHOLE) return 0;
-    if (!(a.flags & GF_KEPT_SPLIT) && !(s.coreLoops < 256u || (s.coreLoops <= 512u && kSteps <= 64u))) return 0;
+    if (!(a.flags & GF_KEPT_SPLIT) && !(s.coreLoops < 256u || (s.coreLoops <= 512u && kSteps <= 80u))) return 0;
     return xcd_uniform_kept(s, a.keptRank);
 }
 

@@ -536,7 +536,7 @@ def test_task_tiles_batch_query_equals_single_queries(so):
 
 def test_kept_split_choice_by_tile_count_and_k_length():
     # which reduce-scatter launches run their kept tiles as two 64-row workgroups (catcoc_kept_split_tiles): fewer than 256
-    # tiles, or up to 512 tiles with up to 64 k steps of 64 bytes; whole tiles, A as [m,k], XCD-block order; flags override
+    # tiles, or up to 512 tiles with up to 80 k steps of 64 bytes; whole tiles, A as [m,k], XCD-block order; flags override
     from mm_rs_with_catlass_amd import ops
     so = L.load()
 
@@ -555,11 +555,11 @@ def test_kept_split_choice_by_tile_count_and_k_length():
     assert split(Q, L.INT8, 4096, 1792, 4096, 8, ta=1) == 0           # A as [k,m]: whole tiles only
     assert split(Q, L.INT8, 4096, 1792, 4096, 8, L.FLAG_KEPT_WHOLE) == 0
     assert split(Q, L.INT8, 4096, 1792, 4096, 8, L.FLAG_LINEAR_ORDER) == 0
-    assert split(Q, L.INT8, 4096, 4096, 4096, 8) == 64                # 64 k steps
-    assert split(Q, L.INT8, 4096, 4160, 4096, 8) == 0                 # 65
+    assert split(Q, L.INT8, 4096, 5120, 4096, 8) == 64                # 80 k steps
+    assert split(Q, L.INT8, 4096, 5184, 4096, 8) == 0                 # 81
     assert split(Q, L.INT8, 1024, 7168, 4096, 8) == 16                # 128 tiles: fewer than CUs, any k
     assert split(RS, L.FP16, 4096, 1792, 4096, 8) == 64               # config 3: 512 tiles, 56 k steps
-    assert split(RS, L.FP16, 4096, 2112, 4096, 8) == 0                # 66 k steps
+    assert split(RS, L.FP16, 4096, 2592, 4096, 8) == 0                # 81 k steps
 
     # the tiles by which tasks + kept halves exceed the 512 workgroup slots run as halves too (catcoc_tail_split_tiles); their
     # checksum halves need the counter block of a workspace
