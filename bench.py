@@ -249,7 +249,7 @@ def tiling_sweep(args, torch, L, ops, dev):
                                                      checksum=csf, out=out)
         rows_all += tuning.sweep_shape("MatmulReduceScatter", mk_float, M, K, N, P, ta, tb, PEAK_F16_TFLOPS, full_tiles=full, progress=progress)
         del A, B, peers
-    path = args.csv or os.path.join(ROOT, "gpurun_out", "result.csv")
+    path = os.path.abspath(args.csv or "result.csv")   # (the reference writes result.csv into the working directory too)
     os.makedirs(os.path.dirname(path), exist_ok=True)
     tuning.write_result_csv(path, rows_all)
     best = tuning.best_results(rows_all)
@@ -415,7 +415,7 @@ def main():
     ap.add_argument("--sustained", type=int, default=300, help="launches of the untimed sustained block (0 = skip)")
     ap.add_argument("--no-other-mode", action="store_true", help="skip the secondary run of the other store mode")
     ap.add_argument("--ceiling-steps", type=int, default=20000, help="--mode ceiling: k steps per launch of the probe")
-    ap.add_argument("--csv", default="", help="--mode sweep: where result.csv goes (default gpurun_out/result.csv)")
+    ap.add_argument("--csv", default="", help="--mode sweep: where result.csv goes (default: result.csv in the working directory)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (peers are staged in the same GPU's HBM); --gpus %d is not "
