@@ -1220,28 +1220,45 @@ def test_launches_replay_from_a_hip_graph():
     assert fac == 4
     ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
     small, out_small = ops.prepare_quant_matmul_splitk(xs, w, ss, s2, None, pk, P, 4, 2, split_k=4, workspace=ws)
-    big(); small(); L.check()
+    # a launch of 512 tiles with split kept tiles, whose waiting tiles run as halves: their checksum halves meet through
+    # the counter block of a workspace and clear it again
+    xh = torch.randint(-127, 128, (4096, 128), dtype=torch.int8, device=DEV, generator=g)
+    wh = torch.randint(-127, 128, (128, 4096), dtype=torch.int8, device=DEV, generator=g)
+    sh1 = torch.empty(4096, device=DEV).uniform_(0.005, 0.02, generator=g)
+    sh2 = torch.empty(4096, device=DEV).uniform_(0.001, 0.01, generator=g)
+    ph = [torch.randn((512, 4096), device=DEV, generator=g) for _ in range(7)]
+    csh = torch.zeros(512, dtype=torch.int64, device=DEV)
+    wsh = torch.zeros(65536, dtype=torch.uint8, device=DEV)
+    halves, out_halves = ops.prepare_quant_matmul_reduce_scatter(xh, wh, sh1, sh2, None, ph, 3, 8, checksum=csh, workspace=wsh)
+    big(); small(); halves(); L.check()
     torch.cuda.synchronize()
-    want_big, want_small = out_big.clone(), out_small.clone()
+    want_big, want_small, want_halves, want_cs = out_big.clone(), out_small.clone(), out_halves.clone(), csh.clone()
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
-        big(); small()                       # warm the side stream before capture
+        big(); small(); halves()             # warm the side stream before capture
         torch.cuda.synchronize()
         with torch.cuda.graph(graph, stream=side):
             out_big.zero_()
             out_small.zero_()
+            out_halves.zero_()
+            csh.zero_()
             big()
             small()
+            halves()
     L.check()
     for _ in range(3):
         out_big.fill_(1.0)                   # eager work between the replays
         out_small.fill_(1.0)
+        out_halves.fill_(1.0)
+        csh.fill_(7)
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out_big, want_big) and torch.equal(out_small, want_small)
+        assert torch.equal(out_halves, want_halves) and torch.equal(csh, want_cs)
         assert not ws[:65536].any(), "tile counters were not re-armed"
+        assert not wsh.any(), "the words the checksum halves meet through were not cleared"
 
 
 def test_cpp_host_drives_the_library_through_the_c_abi(tmp_path):
