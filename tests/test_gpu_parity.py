@@ -1199,6 +1199,38 @@ def test_quant_config5_full_size(M):
     assert np.array_equal(host16(out), want), "kept rows differ from the oracle"
 
 
+@pytest.mark.parametrize("case", [(1024, 16, 0, 64), (512, 8, 448, 64), (768, 3, 256, 96)])
+def test_quant_explicit_kept_rows_large_tiles_streamed_operands(case):
+    """Explicit kept rows on the 128x256 tiles with operands that stream from HBM (K = N = 8192): six-stage ring, the peers'
+    partials in row layout through the ring of register buffers -- with 15, 7 and 2 peers, kept rows at the start, at the end
+    and in the middle of A, whole tiles and k slices.  Kept rows bit for bit against the oracle, the other rows through the
+    per-block checksums."""
+    _need_gpu()
+    M, P, kb, kr = case
+    K = N = 8192
+    g = torch.Generator(device=DEV).manual_seed(900 + M)
+    x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
+    x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=DEV, generator=g)
+    s1 = torch.empty(M, device=DEV).uniform_(0.005, 0.02, generator=g)
+    s2 = torch.empty(N, device=DEV).uniform_(0.001, 0.01, generator=g)
+    peers = [torch.randn((kr, N), device=DEV, generator=g) for _ in range(P - 1)]
+    need, f, blocks = ops.splitk_plan(M, K, N, P, kb, kr, n0=256)
+    ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=DEV)
+    cs = torch.zeros(blocks, dtype=torch.int64, device=DEV)
+    out = ops.quant_matmul_splitk(x1, x2, s1, s2, None, peers, P, kb, kr, workspace=ws, checksum=cs, n0=256)
+    torch.cuda.synchronize()
+    acc_k, want = oracle.quant_matmul_reduce_scatter(x1[kb:kb + kr].cpu().numpy(), x2.cpu().numpy(), s1[kb:kb + kr].cpu().numpy(),
+                                                     s2.cpu().numpy(), None, 0, kr, [p.cpu().numpy() for p in peers], oracle.BF16)
+    assert np.array_equal(host16(out), want), "kept rows differ from the oracle"
+    # rows that are not kept, per 128 x 128 block: exact through row sums of A against column blocks of B
+    notkept = torch.ones(M, dtype=torch.float64, device=DEV)
+    notkept[kb:kb + kr] = 0
+    a_blocks = (x1.double() * notkept[:, None]).view(M // 128, 128, K).sum(1)            # [M/128, K]
+    want_cs = (a_blocks @ x2.double()).view(M // 128, N // 128, 128).sum(2)              # [M/128, N/128]
+    assert torch.equal(cs.view(M // 128, N // 128), want_cs.to(torch.int64))
+    assert not ws[:65536].any()
+
+
 # ------------------------------------------------------- C ABI from a plain C++ host
 def test_launches_replay_from_a_hip_graph():
     # serving loops capture their launches: the library allocates nothing and never synchronises, the split-K path
