@@ -28,9 +28,12 @@ namespace catcoc {
 
 // MBW: 32-row blocks staged per tile (1, 2 or 4); rows past the end of A are clamped to the last row
 // on the way in and masked on the way out.
-template <int MBW>
+// AP: A is fetched per group of two k steps, 128 bytes per row (whole cache lines: half as many requests to L2 as two
+// 64-byte halves), into one "pair" area per group; for 64- and 128-row tiles whose k slices are whole pairs of steps.
+template <int MBW, bool AP = false>
 __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args)
 {
+    static_assert(!AP || MBW >= 2, "pairs of steps are the groups of the 64- and 128-row tiles");
     constexpr int NW = 4;
     constexpr int G = (MBW == 1) ? 4 : 2;      // k steps per barrier
     constexpr int NS = (MBW == 1) ? 12 : 8;    // LDS stages (a multiple of G, at least 2G)
@@ -68,7 +71,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     // power of two apart, so those reads would all queue at one L2 channel.  Each workgroup therefore walks its k
     // steps from a different starting point (integer sums do not care about the order); workgroups that share an
     // XCD (blockIdx mod 8) get consecutive starting points, which spreads them over the channels.
-    const uint32_t rot = (blockIdx.x >> 3) % nsteps;
+    const uint32_t rot = AP ? 2u * ((blockIdx.x >> 3) % (nsteps / 2u)) : (blockIdx.x >> 3) % nsteps;
     auto issue = [&](uint32_t st, uint32_t step) {
         unsigned char *sa = smem + st * STAGE, *sb = sa + A_STAGE;
         const uint32_t kt = step + rot < nsteps ? step + rot : step + rot - nsteps;
@@ -87,6 +90,40 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
             const int j = w + NW * jj;
             const int row = 8 * j + (lane >> 3);
             dma16_stream(Bgk + (size_t)row * ldb + (((lane & 7) ^ (((row >> 1) & 3) << 1)) * 16), sb + j * 1024);
+        }
+    };
+    // AP: steps `step` and `step + 1` (st even).  The group's area holds the pair of A first (rows of 128 bytes: copy j covers
+    // rows 8j..8j+7, lane -> row 8j + lane/8, chunk slot lane&7 holds k chunk slot ^ ((row>>1)&7)), then B of the two steps.
+    auto issue_pair = [&](uint32_t st, uint32_t step) {
+        unsigned char *sp = smem + st * STAGE;
+        const uint32_t kt = step + rot < nsteps ? step + rot : step + rot - nsteps;
+        const unsigned char *Agk = Ag + (size_t)kt * 64;
+#pragma unroll
+        for (int jj = 0; jj < MBW; ++jj) {
+            const int j = w + NW * jj;
+            const uint32_t lrow = 8 * j + (lane >> 3);
+            const uint32_t srow = umin(lrow, rowsValid - 1u);
+            dma16(Agk + (size_t)srow * lda + (((lane & 7) ^ ((lrow >> 1) & 7)) * 16), sp + j * 1024);
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const unsigned char *Bgk = Bg + (size_t)(kt + t) * 64 * ldb;
+            unsigned char *sb = sp + 2 * A_STAGE + t * B_STAGE;
+#pragma unroll
+            for (int jj = 0; jj < B_CP; ++jj) {
+                const int j = w + NW * jj;
+                const int row = 8 * j + (lane >> 3);
+                dma16_stream(Bgk + (size_t)row * ldb + (((lane & 7) ^ (((row >> 1) & 3) << 1)) * 16), sb + j * 1024);
+            }
+        }
+    };
+    auto issue_more = [&](uint32_t &issuedSteps) {   // the next step, or the next pair of steps
+        if constexpr (AP) {
+            issue_pair(issuedSteps % NS, issuedSteps);
+            issuedSteps += 2;
+        } else {
+            issue(issuedSteps % NS, issuedSteps);
+            ++issuedSteps;
         }
     };
 
@@ -171,6 +208,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
 
     const uint32_t a_lds = c32 * 64;
     const uint32_t a_sw = (c32 >> 2) & 3;
+    const uint32_t ap_lds = c32 * 128, ap_sw = (c32 >> 1) & 7;   // pair area: rows of 128 bytes
     // transpose read of this wave's 32 columns (two 16-column chunks, one per half of a 32-lane group)
     const int ti16 = lane & 15, tch = (lane >> 4) & 1, trow = ti16 >> 1, thalf = ti16 & 1;
     const uint32_t b_lds = (16 * h + trow) * 128 + (((2 * w + tch) ^ (((trow >> 1) & 3) << 1)) * 16) + thalf * 8;
@@ -178,8 +216,9 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     // The loop is paced by latencies, not by bandwidth (one wave per SIMD: barrier, LDS round trip and the MFMA
     // chain of a step add up), so G steps share one barrier and one LDS round trip.  `issued` counts the steps
     // whose copies have been issued; before a group is read, the copies of later steps may stay in flight.
-    uint32_t issued = umin(nsteps, (uint32_t)(NS - G));
-    for (uint32_t i = 0; i < issued; ++i) issue(i, i);
+    const uint32_t ahead = umin(nsteps, (uint32_t)(NS - G));
+    uint32_t issued = 0;
+    while (issued < ahead) issue_more(issued);
     auto wait_steps_in_flight = [&](uint32_t n) {
         switch (n) {
             case 0: CATCOC_WAIT_VMCNT(0); break;
@@ -199,16 +238,15 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         wait_steps_in_flight(issued - (s + GG));
         barrier_keep_vmem();
         // every wave has left the steps before s: their stages take the next copies
-        while (issued < nsteps && issued < s + NS) {
-            issue(issued % NS, issued);
-            ++issued;
-        }
+        while (issued < nsteps && issued < s + NS) issue_more(issued);
         // all fragment reads of the group first, then the MFMAs: one LDS round trip per group (left to itself the
         // compiler reuses two fragment registers and serialises them)
         v4i bf[GG][2], af[GG][2][MBW];
 #pragma unroll
         for (int j = 0; j < GG; ++j) {
-            const unsigned char *sa = smem + ((s + j) % NS) * STAGE, *sb = sa + A_STAGE;
+            // (AP: the group's area starts at the stage of its first step: the pair of A, then B of step j)
+            const unsigned char *sa = AP ? smem + (s % NS) * STAGE : smem + ((s + j) % NS) * STAGE;
+            const unsigned char *sb = AP ? sa + 2 * A_STAGE + j * B_STAGE : sa + A_STAGE;
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
                 const unsigned char *p = sb + b_lds + kk * 32 * 128;
@@ -216,8 +254,10 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
                 const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 128));
                 bf[j][kk] = v4i{t0.x, t0.y, t1.x, t1.y};
 #pragma unroll
-                for (int mb = 0; mb < MBW; ++mb)
-                    af[j][kk][mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
+                for (int mb = 0; mb < MBW; ++mb) {
+                    if constexpr (AP) af[j][kk][mb] = *(const v4i *)(sa + ap_lds + mb * 32 * 128 + (((4 * j + 2 * kk + h) ^ ap_sw) * 16));
+                    else af[j][kk][mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
+                }
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -236,9 +276,12 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     for (; issued < nsteps && s + G <= nsteps; s += G) k_group(s, std::integral_constant<int, G>{});
     request_epilogue_operands();
     for (; s + G <= nsteps; s += G) k_group(s, std::integral_constant<int, G>{});
-    for (; s < nsteps; ++s) k_group(s, std::integral_constant<int, 1>{});
+    if constexpr (!AP) {   // (with pairs the host guarantees whole groups)
+        for (; s < nsteps; ++s) k_group(s, std::integral_constant<int, 1>{});
+    }
 
     // ---- k slices meet -------------------------------------------------------------
+    long long csumOthers = 0;   // what the other slices hold of the groups that did not travel (checksums only)
     if (f > 1) {
         // Partial tiles travel through memory at device scope (cache policy sc1: written through / read past
         // the XCD-local L2), as ordinary buffer accesses so that the loads of a slice are issued together.  Inside
@@ -248,10 +291,12 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         constexpr int DEVICE_SCOPE = 16;   // sc1
         const size_t tileBytes = 128 * 128 * 4;
         // A group of eight rows travels when it has rows of A and somebody will look at them: kept rows (the output), or
-        // every row when the caller asked for checksums or a dump of the accumulators.  With neither, the partials of rows
-        // that are not kept are dropped where they are: at M = 128 with 16 kept rows a workgroup publishes 8 KiB instead of
-        // 64, and the last slice fetches 24 KiB instead of 192.
-        const bool allRows = args.checksum != nullptr || args.accDump != nullptr;
+        // every row when the caller asked for a dump of the accumulators.  The partials of the other groups stay where
+        // they are: at M = 128 with 16 kept rows a workgroup publishes 8 KiB instead of 64, and the last slice fetches
+        // 24 KiB instead of 192.  A checksum needs only their sum, and sums of sums are exact: every lane adds up what
+        // it holds of those groups and the eight bytes travel in the place of the first group that stays behind.
+        // (Tiles of up to 32 rows have four groups at most: there every row travels when checksums are asked for.)
+        const bool allRows = args.accDump != nullptr || (MBW == 1 && args.checksum != nullptr);
         auto group_valid = [&](int mb, int g) {   // wave-uniform
             const uint32_t g0 = (uint32_t)(mb * 32 + g * 8);
             if (g0 >= rowsValid) return false;
@@ -259,6 +304,24 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         };
         const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
             (void *)(args.skPart + ((size_t)slice * loopsM * loopsN + tile) * (128 * 128)), 0, (int)tileBytes, 0x00020000);
+        int sumSlot = -1;   // first group with rows of A that does not travel (wave-uniform)
+        long long behind = 0;
+        if (MBW >= 2 && args.checksum != nullptr) {
+#pragma unroll
+            for (int mb = MBW - 1; mb >= 0; --mb)
+#pragma unroll
+                for (int g = 3; g >= 0; --g)
+                    if ((uint32_t)(mb * 32 + g * 8) < rowsValid && !group_valid(mb, g)) {
+                        sumSlot = mb * 4 + g;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            behind += (uint32_t)(mb * 32 + g * 8 + j) + 4u * h < rowsValid ? acc[mb][4 * g + j] : 0;
+                    }
+            if (sumSlot >= 0) {
+                const v2i sv = {(int)(uint32_t)(unsigned long long)behind, (int)(uint32_t)((unsigned long long)behind >> 32)};
+                __builtin_amdgcn_raw_buffer_store_b64(sv, mine, (sumSlot * 256 + tid) * 16, 0, DEVICE_SCOPE);
+            }
+        }
 #pragma unroll
         for (int mb = 0; mb < MBW; ++mb)
 #pragma unroll
@@ -281,6 +344,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         constexpr int QG = 3;
         for (uint32_t o0 = 0; o0 + 1 < f; o0 += QG) {
             v4i pv[QG][MBW][4];
+            v2i sums[QG];
 #pragma unroll
             for (int q = 0; q < QG; ++q) {
                 const uint32_t o = o0 + q;                       // o-th of the f - 1 other slices
@@ -288,6 +352,8 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
                 const uint32_t sl = o < slice ? o : o + 1;
                 const __amdgpu_buffer_rsrc_t other = __builtin_amdgcn_make_buffer_rsrc(
                     (void *)(tile0 + (use ? sl : slice) * sliceStride), 0, use ? (int)tileBytes : 0, 0x00020000);
+                sums[q] = v2i{0, 0};
+                if (use && sumSlot >= 0) sums[q] = __builtin_amdgcn_raw_buffer_load_b64(other, (sumSlot * 256 + tid) * 16, 0, DEVICE_SCOPE);
 #pragma unroll
                 for (int mb = 0; mb < MBW; ++mb)
 #pragma unroll
@@ -298,7 +364,8 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
                     }
             }
 #pragma unroll
-            for (int q = 0; q < QG; ++q)
+            for (int q = 0; q < QG; ++q) {
+                csumOthers += (long long)(((unsigned long long)(uint32_t)sums[q].y << 32) | (uint32_t)sums[q].x);
 #pragma unroll
                 for (int mb = 0; mb < MBW; ++mb)
 #pragma unroll
@@ -308,6 +375,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
                         acc[mb][4 * g + 2] += pv[q][mb][g].z;
                         acc[mb][4 * g + 3] += pv[q][mb][g].w;
                     }
+            }
         }
     }
 
@@ -317,7 +385,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     // block it was several times the size of the instruction cache): the block's registers are selected, dequantised,
     // the peers added in slot order eight at a time (the first block's first eight are in registers already, the
     // others are fetched into the same registers in one round trip) and the 16-bit rows stored.
-    long long csum = 0;
+    long long csum = csumOthers;
 #pragma unroll
     for (int mb = 0; mb < MBW; ++mb) {
         if ((uint32_t)mb * 32 >= rowsValid) break;

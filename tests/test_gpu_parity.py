@@ -449,6 +449,45 @@ def test_quant_skinny_m_splitk(case):
         assert cs[t] == blk[~keep[mi * 128:(mi + 1) * 128]].sum(), t
 
 
+@pytest.mark.parametrize("case", [(64, 256, 4096, 8, 8, 8, 0), (128, 640, 2048, 8, 112, 16, 0), (200, 256, 1088, 4, 100, 50, 3),
+                                  (100, 384, 1024, 8, 37, 13, 4), (256, 256, 2048, 2, 130, 60, 2), (33, 128, 512, 2, 0, 33, 2),
+                                  (128, 256, 1024, 1, 0, 128, 4), (190, 128, 768, 8, 0, 5, 3)])
+def test_quant_skinny_m_splitk_checksums_without_dump(case):
+    """Checksums without a dump of the accumulators: the k slices then hand over only the groups of eight rows that hold kept
+    rows, and every lane's sum of what it holds of the other groups.  Kept ranges that start and end inside a group, rows
+    of A that end inside a group, every row kept, k slices of an odd number of steps: the checksum of every tile equals the
+    oracle's sum over the rows that are not kept, the kept rows its output, on two launches through one workspace."""
+    _need_gpu()
+    M, N, K, P, kb, kr, f = case
+    rng = np.random.default_rng(160 + M)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.integers(-1000, 1000, N, dtype=np.int32)
+    peers = [rng.standard_normal((kr, N)).astype(np.float32) for _ in range(P - 1)]
+    acc_want, out_want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, b, kb, kr, peers, oracle.BF16)
+    need, fac, tiles = ops.splitk_plan(M, K, N, P, kb, kr, split_k=f, n0=128)
+    ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=DEV)
+    checksum = torch.zeros(tiles, dtype=torch.int64, device=DEV)
+    launch, out = ops.prepare_quant_matmul_splitk(dev(x1), dev(x2), dev(s1), dev(s2), dev(b), [dev(p) for p in peers], P,
+                                                  kb, kr, split_k=f, workspace=ws, checksum=checksum, n0=128)
+    keep = np.zeros(M, bool)
+    keep[kb:kb + kr] = True
+    for it in range(2):
+        out.zero_()
+        checksum.fill_(-1)
+        launch()
+        L.check()
+        torch.cuda.synchronize()
+        assert np.array_equal(host16(out), out_want), "kept rows differ from the oracle"
+        cs = checksum.cpu().numpy()
+        for t in range(tiles):
+            mi, ni = divmod(t, N // 128)
+            blk = acc_want[mi * 128:(mi + 1) * 128, ni * 128:(ni + 1) * 128].astype(np.int64)
+            assert cs[t] == blk[~keep[mi * 128:(mi + 1) * 128]].sum(), (it, t)
+
+
 def test_quant_skinny_m_rejections():
     _need_gpu()
     x1 = torch.zeros((16, 96), dtype=torch.int8, device=DEV)
