@@ -302,7 +302,8 @@ struct SplitkPlan {
 // workspace) when the shape has full tiles and the kept rows are whole 32-row blocks.  Such launches have at most one
 // workgroup per CU and run the kernel's six-stage ring with the pipelined peer loads.  Measured at K = N = 8192 with kept
 // rows = M / 8, the two routes alternating launch by launch and B coming from HBM (six copies, another one every launch):
-// M = 1024 106 against 166 us, M = 512 69 (two k slices) against 77 us, M = 256 50 (four k slices) against 48 us.  n0 = 256
+// M = 1024 106 against 166 us, M = 512 69 (two k slices) against 77 us, M = 256 50 (four k slices) against 48 us (since then
+// both routes fetch A as whole cache lines per pair of k steps, which took 4 to 7 us off each of these).  n0 = 256
 // (with m0 0 or 128) in the tiling asks for the large tile explicitly, n0 = 128 for the split-K kernel.
 constexpr uint32_t kLargeTileRows = 512;
 

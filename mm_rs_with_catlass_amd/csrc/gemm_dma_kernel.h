@@ -79,12 +79,19 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 //   128-row tile: three A stages (8 KiB each), then three B stages (16 KiB each)            = 72 KiB
 //   256-row tile: two A pair buffers (32 KiB each), then four B stages (16 KiB each)         = 128 KiB
 // (a 64-row tile of the four-wave geometry uses the first 60 KiB of the 72)
-template <int WM, int NS = 3> struct DmaPool { static constexpr int BYTES = (WM == 4) ? (4 * 256 * 64 + 4 * 64 * 256) : NS * (128 * 64 + 64 * 256); };
+//   128-row tile, six stages, A in pairs (AQ): four A pair buffers (16 KiB each), then six B stages = 160 KiB, the whole LDS
+template <int WM, int NS = 3, bool AQ = false> struct DmaPool
+{
+    static constexpr int BYTES = (WM == 4) ? (4 * 256 * 64 + 4 * 64 * 256) : AQ ? ((NS / 2 + 1) * 128 * 128 + NS * 64 * 256) : NS * (128 * 64 + 64 * 256);
+};
 
 // One tile (or one k slice of a tile) of the launch: position `pos` of the launch order, in the caller's LDS pool.
 // MB = 32-row blocks per wave (2; 1 = a 64-row tile, four-wave geometry only); subRow = first row of a 64-row tile inside
 // its 128-row tile of the schedule.
-template <uint32_t DT, int WM, bool TB, bool RM, bool RG, bool TA, int MB, int NS = 3, bool PP = false>
+// AQ = A is copied per pair of k steps, 128 bytes per row (whole cache lines: half as many requests to L2 as two 64-byte
+// halves), as the 256-row geometry does; for the six-stage ring, whose launches have one workgroup per CU and feel every
+// request (with three stages and two workgroups per CU the same change measured slower).
+template <uint32_t DT, int WM, bool TB, bool RM, bool RG, bool TA, int MB, int NS = 3, bool PP = false, bool AQ = false>
 __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *smem, uint32_t pos, uint32_t slice, uint32_t kSlices,
                                          uint32_t subRow)
 {
@@ -94,6 +101,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     static_assert(WM == 2 || WM == 4, "supported geometries");
     static_assert(NS == 3 || (WM == 2 && NS >= 3 && NS <= 8), "deeper rings exist for the 128-row kernel");
     static_assert(MB == 2 || (MB == 1 && WM == 2 && !RM && !RG && !TA), "64-row tiles exist for the four-wave geometry with A as [m,k]");
+    static_assert(!AQ || (WM == 2 && NS == 6 && MB == 2 && !TA), "pairs of A steps exist for the six-stage 128-row kernel with A as [m,k]");
     using Acc = typename AccOf<DT>::type;
     constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
     constexpr int NW = 2 * WM;          // waves
@@ -103,7 +111,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     constexpr int A_DMA = BM / 16 / NW;  // 1 KiB copies per wave per stage
     constexpr int B_DMA = 16 / NW;
     constexpr int STEP_DMA = A_DMA + B_DMA;
-    constexpr int POOL = DmaPool<WM, NS>::BYTES;
+    constexpr int POOL = DmaPool<WM, NS, AQ>::BYTES;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -373,7 +381,108 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
 #undef CATCOC_MMA
     auto nothing = [] {};
 
-    if constexpr (WM == 2) {
+    if constexpr (WM == 2 && AQ) {
+        // ---- NS B stages, NS / 2 + 1 A pair buffers.  B runs NS - 1 steps ahead as in the plain ring; pair q (steps 2q,
+        // 2q + 1) is issued at step 2q - NS into buffer q mod (NS / 2 + 1), which pair q - NS / 2 - 1 left before that
+        // step's barrier.  Copies a wave issues in step kt, in this order: B(kt + NS - 1), then on even kt the pair
+        // (kt + NS) / 2; the prologue issues what the steps -NS .. -1 would have.  The vector-memory counter retires in
+        // order, so at the barrier of step s everything issued after B(s) may still be in flight: the B copies of the NS - 2
+        // steps after s and the pairs issued at the even steps s - (NS - 1) .. s - 1 (three of them when s is odd, two when
+        // it is even), fewer towards the end of the k range.  A pair and a B step are the same number of copies per wave.
+        constexpr int NPB = NS / 2 + 1;
+        constexpr int AP = BM * 128;
+        constexpr int APC = BM / 8 / NW;
+        static_assert(APC == B_DMA, "the waits count pairs and B steps in one unit");
+        static_assert(NPB * AP + NS * B_STAGE <= POOL, "pair buffers and B stages fit the pool");
+        static_assert((NS - 2 + NS / 2) * B_DMA <= 63, "the wait counter holds 63");
+        auto stB = [&](uint32_t st) { return smem + NPB * AP + st * B_STAGE; };
+        auto offB = [&](uint32_t st) { return NPB * AP + st * B_STAGE; };
+        // pair copy j covers rows 8j..8j+7: lane -> row 8j + lane/8, slot lane&7 holds chunk slot ^ ((row>>1)&7)
+        const unsigned char *gP[APC];
+#pragma unroll
+        for (int jj = 0; jj < APC; ++jj) {
+            const int row = 8 * (w + NW * jj) + (lane >> 3);
+            gP[jj] = Ag + (size_t)row * ldaB + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+        }
+        auto issue_ap = [&](uint32_t q) {   // pairs are issued in increasing q
+#pragma unroll
+            for (int jj = 0; jj < APC; ++jj) {
+                dma16_at(gP[jj], lds0 + (q % NPB) * AP + (ws + NW * jj) * 1024);
+                gP[jj] += 128;
+            }
+        };
+        const uint32_t ap_lds = (wm * 32 * MB + c32) * 128;
+        const uint32_t ap_sw = (c32 >> 1) & 7;
+        auto load_ap = [&](v4i (&af)[MB], uint32_t kt, int kk) {
+            const unsigned char *sa = smem + ((kt >> 1) % NPB) * AP + ap_lds + ((((kt & 1) * 4 + 2 * kk + h) ^ ap_sw) * 16);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) af[mb] = *(const v4i *)(sa + mb * 32 * 128);
+        };
+        auto wait_units = [&](uint32_t n) {   // at most n x B_DMA copies (the youngest) outstanding
+            switch (n) {
+                case 0: CATCOC_WAIT_VMCNT(0); break;
+                case 1: CATCOC_WAIT_VMCNT(1 * B_DMA); break;
+                case 2: CATCOC_WAIT_VMCNT(2 * B_DMA); break;
+                case 3: CATCOC_WAIT_VMCNT(3 * B_DMA); break;
+                case 4: CATCOC_WAIT_VMCNT(4 * B_DMA); break;
+                case 5: CATCOC_WAIT_VMCNT(5 * B_DMA); break;
+                case 6: CATCOC_WAIT_VMCNT(6 * B_DMA); break;
+                default: CATCOC_WAIT_VMCNT(7 * B_DMA); break;
+            }
+        };
+        auto units_after = [&](uint32_t s) {   // B steps and pairs issued after B(s) by the time step s starts
+            const uint32_t nB = umin((uint32_t)(NS - 2), nk - 1u - s);
+            // pairs: issued at the even (possibly virtual, negative) steps t with s - (NS - 1) <= t <= min(s - 1, nk - NS - 2);
+            // counted with t shifted by NS + 2, which keeps the parity and makes every term non-negative
+            const uint32_t lo = s + 3u, hiA = s + (uint32_t)NS + 1u, hiB = nk;
+            const uint32_t hi = umin(hiA, hiB);
+            const uint32_t nP = hi >= lo ? (hi >> 1) - ((lo + 1u) >> 1) + 1u : 0u;
+            return nB + nP;
+        };
+        // the prologue: what the steps -NS .. -1 would have issued
+#pragma unroll
+        for (int v = -NS; v < 0; ++v) {
+            if (v + NS - 1 >= 0 && (uint32_t)(v + NS - 1) < nk) issue_b(offB(v + NS - 1));
+            if ((v & 1) == 0 && (uint32_t)(v + NS + 2) <= nk) issue_ap((uint32_t)(v + NS) >> 1);
+        }
+        // step 0 (peeled: no MFMAs pending yet)
+        wait_units(units_after(0));
+        barrier_keep_vmem();
+        if ((uint32_t)(NS - 1) < nk) issue_b(offB(NS - 1));
+        if ((uint32_t)(NS + 2) <= nk) issue_ap(NS >> 1);
+        load_ap(fa0, 0, 0);
+        load_b(fb0, stB(0), 0);
+        load_ap(fa1, 0, 1);
+        load_b(fb1, stB(0), 1);
+        CATCOC_FENCE();
+        mma(fa0, fb0);
+        CATCOC_FENCE();
+        // step kt reads B stage kt % NS and refills stage (kt - 1) % NS with B(kt + NS - 1)
+        uint32_t kt = 1, cur = 1, nxt = 0;
+        auto step = [&]() {
+            const uint32_t k = kt;
+            const bool moreB = k + (uint32_t)(NS - 1) < nk, moreP = (k & 1u) == 0 && k + (uint32_t)(NS + 2) <= nk;
+            sched_step([&](v4i (&af)[MB], int kk) { load_ap(af, k, kk); }, stB(cur), [&] { if (moreB) issue_b(offB(nxt)); },
+                       [&] { if (moreP) issue_ap((k + (uint32_t)NS) >> 1); }, nothing, nothing);
+            ++kt;
+            cur = cur == NS - 1 ? 0 : cur + 1;
+            nxt = nxt == NS - 1 ? 0 : nxt + 1;
+        };
+        while (kt + (uint32_t)(NS + 2) <= nk) {   // kt is odd here: an odd and an even step in full flight
+            CATCOC_WAIT_VMCNT((NS - 2 + NS / 2) * B_DMA);
+            barrier_keep_vmem();
+            step();
+            CATCOC_WAIT_VMCNT((NS - 3 + NS / 2) * B_DMA);
+            barrier_keep_vmem();
+            step();
+        }
+        while (kt < nk) {
+            wait_units(units_after(kt));
+            barrier_keep_vmem();
+            step();
+        }
+        mma(fa1, fb1);
+    } else if constexpr (WM == 2) {
         // ---- NS stages, copies run NS - 1 k steps ahead.  NS = 3: 72 KiB LDS, two workgroups per CU, for operands that come
         // out of L2 or the Infinity Cache.  NS = 6: 144 KiB, one workgroup per CU, 120 KiB in flight per CU: for launches of at
         // most one workgroup per CU anyway, whose operands stream from HBM (two steps ahead do not cover that latency) ----
@@ -1074,10 +1183,10 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
 }
 
 // One workgroup per tile, or per k slice of a tile.
-template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false, int NS = 3, bool PP = false>
+template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false, int NS = 3, bool PP = false, bool AQ = false>
 __global__ void __launch_bounds__(128 * WM, NS == 3 ? 2 : 1) gemm_dma_kernel(const GemmArgs args)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<WM, NS>::BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<WM, NS, AQ>::BYTES];
     // A launch with few tiles can cut every tile's k range into kSlices pieces, one workgroup each (128-row tiles
     // only): position `pos` of the launch order runs as kSlices workgroups that stay in the position's XCD column.
     uint32_t pos = blockIdx.x + args.taskBase, slice = 0;   // (taskBase is zero for k-sliced launches)
@@ -1092,7 +1201,7 @@ __global__ void __launch_bounds__(128 * WM, NS == 3 ? 2 : 1) gemm_dma_kernel(con
             pos = blockIdx.x / kSlices;
         }
     }
-    dma_tile<DT, WM, TB, RM, RG, TA, 2, NS, PP>(args, smem, pos, slice, kSlices, 0);
+    dma_tile<DT, WM, TB, RM, RG, TA, 2, NS, PP, AQ>(args, smem, pos, slice, kSlices, 0);
 }
 
 // Reduce-scatter launches of a single round of workgroups (no more tiles than the 512 slots of the GPU) run some tiles as two
@@ -1138,6 +1247,15 @@ inline bool deep_ring(const GemmArgs &a, uint32_t workgroups, uint64_t es /* byt
     return workgroups <= 256u && (uint64_t)a.K * es * ((uint64_t)a.M * (a.sched.op == OP_ALLGATHER ? a.sched.P : 1u) + a.N) >= (48ull << 20);
 }
 
+// The six-stage ring copies A in pairs of k steps (whole 128-byte lines per row) when every workgroup's k range is whole
+// pairs and long enough for the ring to fill (A as [m,k]).  Same measurement, both variants alternating: M = 512 (two k
+// slices) 71.2 -> 65.4 us, M = 1024 105.8 -> 98.4 us.
+inline bool deep_ring_pairs(const GemmArgs &a, uint64_t es)
+{
+    const uint64_t nkAll = (uint64_t)a.K * es / 64u, f = a.splitK > 1 ? a.splitK : 1u;
+    return !a.transA && ((uint64_t)a.K * es) % 64u == 0 && nkAll % (2u * f) == 0 && nkAll / f >= 16u;
+}
+
 // Launch of the 128-row geometry: one instantiation per operand layout (A as [m][k] or [k][m], B as [k][n] or [n][k]) and
 // for ragged problems; one workgroup per tile, or per k slice of a tile.
 template <uint32_t DT>
@@ -1152,8 +1270,12 @@ inline int launch_dma_128(const GemmArgs &args, hipStream_t s)
                 hipLaunchKernelGGL((gemm_dma_split_kept_kernel<DT, false>), dim3(args.sched.coreLoops + 8u * (keptPerXcd + tailPerXcd)), block, 0, s, args,
                                    keptPerXcd, tailPerXcd);
             }
-            else if (deep_ring(args, grid.x, DT == DT_I8 ? 1u : 2u))
-                hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false, 6, true>), grid, block, 0, s, args);
+            else if (deep_ring(args, grid.x, DT == DT_I8 ? 1u : 2u)) {
+                if (deep_ring_pairs(args, DT == DT_I8 ? 1u : 2u))
+                    hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false, 6, true, true>), grid, block, 0, s, args);
+                else
+                    hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false, 6, true>), grid, block, 0, s, args);
+            }
             else
                 hipLaunchKernelGGL((gemm_dma_kernel<DT, 2, false, false, false, false>), grid, block, 0, s, args);
             break;

@@ -1238,15 +1238,17 @@ def test_quant_config5_full_size(M):
     assert np.array_equal(host16(out), want), "kept rows differ from the oracle"
 
 
-@pytest.mark.parametrize("case", [(1024, 16, 0, 64), (512, 8, 448, 64), (768, 3, 256, 96)])
+@pytest.mark.parametrize("case", [(1024, 16, 0, 64, 8192), (512, 8, 448, 64, 8192), (768, 3, 256, 96, 8192),
+                                  (128, 4, 64, 32, 8192),      # eight k slices of 16 steps: the shortest range that runs A in pairs
+                                  (1024, 8, 128, 128, 8256)])  # an odd number of k steps: A step by step
 def test_quant_explicit_kept_rows_large_tiles_streamed_operands(case):
     """Explicit kept rows on the 128x256 tiles with operands that stream from HBM (K = N = 8192): six-stage ring, the peers'
-    partials in row layout through the ring of register buffers -- with 15, 7 and 2 peers, kept rows at the start, at the end
-    and in the middle of A, whole tiles and k slices.  Kept rows bit for bit against the oracle, the other rows through the
+    partials in row layout through the ring of register buffers, A copied in pairs of k steps where the k range allows --
+    with 15, 7, 3 and 2 peers, kept rows at the start, at the end and in the middle of A, whole tiles and k slices.  Kept rows bit for bit against the oracle, the other rows through the
     per-block checksums."""
     _need_gpu()
-    M, P, kb, kr = case
-    K = N = 8192
+    M, P, kb, kr, K = case
+    N = 8192
     g = torch.Generator(device=DEV).manual_seed(900 + M)
     x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
     x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=DEV, generator=g)
