@@ -690,6 +690,22 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     // elects the last slice to arrive, and that workgroup adds the others' partials and goes on to the epilogue.
     // Integer partials add exactly in any order; float partials are limited to two slices by the host, whose sum
     // does not depend on which of them arrives last.
+    // RM: only the 32-row blocks with kept rows travel (unless the caller wants a dump of every accumulator): of the others
+    // a checksum needs the sum alone, and sums of sums are exact, so every lane adds up what it holds of such a block and
+    // the eight bytes travel in the place of the block's first 16.  At M = 512 with 64 kept rows three tiles in four then
+    // hand over 4 KiB instead of 128 and the fourth 64 KiB.
+    uint32_t travelMb = (1u << MB) - 1u;   // bit mb: block mb of this wave travels whole (wave-uniform)
+    long long othersSum[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) othersSum[mb] = 0;
+    if constexpr (RM) {
+        if (args.accDump == nullptr) {
+            travelMb = 0;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                if ((ti.row + wm * 32 * MB + mb * 32 - args.keptBegin) < args.keptRows) travelMb |= 1u << mb;
+        }
+    }
     if constexpr (WM == 2) {
         if (kSlices > 1) {
             constexpr int DEVICE_SCOPE = 16;   // sc1
@@ -697,15 +713,28 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
                 (void *)(args.skPart + ((size_t)task * kSlices + slice) * TILE_WORDS), 0, (int)(TILE_WORDS * 4), 0x00020000);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+            for (int mb = 0; mb < MB; ++mb) {
+                if (travelMb & (1u << mb)) {
 #pragma unroll
-                for (int nb = 0; nb < 4; ++nb)
+                    for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const auto e0 = acc[mb][nb][4 * g], e1 = acc[mb][nb][4 * g + 1], e2 = acc[mb][nb][4 * g + 2], e3 = acc[mb][nb][4 * g + 3];
-                        const v4i iv = {__builtin_bit_cast(int, e0), __builtin_bit_cast(int, e1), __builtin_bit_cast(int, e2), __builtin_bit_cast(int, e3)};
-                        __builtin_amdgcn_raw_buffer_store_b128(iv, mine, (((mb * 4 + nb) * 4 + g) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+                        for (int g = 0; g < 4; ++g) {
+                            const auto e0 = acc[mb][nb][4 * g], e1 = acc[mb][nb][4 * g + 1], e2 = acc[mb][nb][4 * g + 2], e3 = acc[mb][nb][4 * g + 3];
+                            const v4i iv = {__builtin_bit_cast(int, e0), __builtin_bit_cast(int, e1), __builtin_bit_cast(int, e2), __builtin_bit_cast(int, e3)};
+                            __builtin_amdgcn_raw_buffer_store_b128(iv, mine, (((mb * 4 + nb) * 4 + g) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+                        }
+                } else if constexpr (RM) {
+                    if (args.checksum != nullptr) {
+                        long long sb = 0;
+#pragma unroll
+                        for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) sb += acc[mb][nb][r];
+                        const v2i sv = {(int)(uint32_t)(unsigned long long)sb, (int)(uint32_t)((unsigned long long)sb >> 32)};
+                        __builtin_amdgcn_raw_buffer_store_b64(sv, mine, ((mb * 16) * 256 + tid) * 16, 0, DEVICE_SCOPE);
                     }
+                }
+            }
             CATCOC_WAIT_VMCNT(0);   // once the stores are acknowledged the slice may be counted
             __syncthreads();
             volatile uint32_t *flag = (volatile uint32_t *)smem;
@@ -719,6 +748,15 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                     (void *)(args.skPart + ((size_t)task * kSlices + sl) * TILE_WORDS), 0, (int)(TILE_WORDS * 4), 0x00020000);
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {   // one 32-row block (64 registers) per round trip
+                    if (!(travelMb & (1u << mb))) {
+                        if constexpr (RM) {
+                            if (args.checksum != nullptr) {
+                                const v2i sv = __builtin_amdgcn_raw_buffer_load_b64(other, ((mb * 16) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+                                othersSum[mb] += (long long)(((unsigned long long)(uint32_t)sv.y << 32) | (uint32_t)sv.x);
+                            }
+                        }
+                        continue;
+                    }
                     v4i pv[4][4];
 #pragma unroll
                     for (int nb = 0; nb < 4; ++nb)
@@ -840,7 +878,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                 for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) sb += acc[mb][nb][r];
-                si += (kept && (keptMb & (1u << mb))) ? 0ll : sb;
+                si += (kept && (keptMb & (1u << mb))) ? 0ll : sb + othersSum[mb];
             }
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) si += __shfl_xor(si, o, 64);
