@@ -303,9 +303,11 @@ struct SplitkPlan {
 // workgroup per CU and run the kernel's six-stage ring with the pipelined peer loads.  Measured at K = N = 8192 with kept
 // rows = M / 8, the two routes alternating launch by launch and B coming from HBM (six copies, another one every launch):
 // M = 1024 106 against 166 us, M = 512 69 (two k slices) against 77 us, M = 256 50 (four k slices) against 48 us (since then
-// both routes fetch A as whole cache lines per pair of k steps, which took 4 to 7 us off each of these).  n0 = 256
+// both routes fetch A as whole cache lines per pair of k steps and hand only kept blocks between k slices: M = 512 59 against 74 us,
+// M = 384 56 against 103 (three rows of 128x128 tiles in four slices are three waves of workgroups), M = 256 42 against 50, and with
+// 32 kept rows M = 128 45 (eight k slices) against 36, so the large tile starts at 256 rows).  n0 = 256
 // (with m0 0 or 128) in the tiling asks for the large tile explicitly, n0 = 128 for the split-K kernel.
-constexpr uint32_t kLargeTileRows = 512;
+constexpr uint32_t kLargeTileRows = 256;
 
 int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uint32_t transA, uint32_t transB, SplitkPlan &sp)
 {

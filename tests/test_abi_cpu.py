@@ -263,10 +263,11 @@ def test_workspace_size_queries(so):
     need, f, tiles = ops.splitk_plan(16, 8192, 8192, 8, 0, 2)
     assert (f, tiles) == (oracle.splitk_factor(16, 8192, 8192, 256, 128, 128, 256), 64)
     assert need == f * tiles * 128 * 128 * 4 + 65536    # counter block of a fixed size first, then the partial tiles
-    # from 512 rows on (full tiles, kept rows in whole 32-row blocks): 128x256 tiles, k slices that fill the CUs once
+    # from 256 rows on (full tiles, kept rows in whole 32-row blocks): 128x256 tiles, k slices that fill the CUs once
     assert ops.splitk_plan(512, 8192, 8192, 8, 0, 64) == (65536 + 128 * 2 * 131072, 2, 256)
-    assert ops.splitk_plan(256, 8192, 8192, 8, 0, 32, n0=256) == (65536 + 64 * 4 * 131072, 4, 128)   # below that on request
-    assert ops.splitk_plan(256, 8192, 8192, 8, 0, 32)[2] == 128 and ops.splitk_plan(256, 8192, 8192, 8, 0, 32)[0] != 65536 + 64 * 4 * 131072
+    assert ops.splitk_plan(256, 8192, 8192, 8, 0, 32) == (65536 + 64 * 4 * 131072, 4, 128)
+    assert ops.splitk_plan(256, 8192, 8192, 8, 0, 32, n0=128)[1:] == (oracle.splitk_factor(256, 8192, 8192, 256, 128, 128, 256), 128)
+    assert ops.splitk_plan(128, 8192, 8192, 4, 0, 32)[0] != 65536 + 32 * 8 * 131072     # below that the split-K kernel, unless asked
     assert ops.splitk_plan(512, 8192, 8192, 8, 0, 64, n0=128) == (0, 1, 256)        # on request: the 128x128 split-K kernel
     assert ops.splitk_plan(512, 8192, 8192, 8, 0, 60)[1:] == (1, 256)               # kept rows not in 32-row blocks: split-K kernel
     assert ops.splitk_plan(1024, 8192, 8192, 8, 0, 128) == (0, 1, 512)              # many rows: 256 tiles of 128x256, no slices
