@@ -155,6 +155,20 @@ def float_configs(args, torch, L, ops, dev):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / args.steps, e0.elapsed_time(e1) / args.steps / 1e3
 
+    def timed_rotating(fns):
+        """The same with another set of operands on every launch (they then come from HBM, not from the Infinity Cache)."""
+        for f in fns:
+            f()
+        L.check()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(args.steps):
+            fns[i % len(fns)]()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps / 1e3
+
     def slices(comm, dt, m, k, n, rank, p):
         """Workspace for a launch of few tiles (the library cuts their k range into slices that meet through it)."""
         need, f = ops.kslice_plan(comm, dt, m, k, n, rank, p)
@@ -171,13 +185,22 @@ def float_configs(args, torch, L, ops, dev):
     out = torch.empty((rows, N), dtype=torch.float16, device=dev)
     ws3 = torch.zeros(65536, dtype=torch.uint8, device=dev)   # counter block: the checksum halves of tiles that run as two workgroups meet here
     wall, kern = timed(lambda: ops.matmul_reduce_scatter(A, B, peers, rank, P, checksum=cs, out=out, workspace=ws3))
+    sets3 = [(A, B, peers)]
+    for _ in range(3):
+        sets3.append((torch.randn((M, K), device=dev, generator=g).half(), (torch.randn((K, N), device=dev, generator=g) * 0.02).half(),
+                      [torch.randn((rows, N), device=dev, generator=g) for _ in range(P - 1)]))
+    out_r = torch.empty((rows, N), dtype=torch.float16, device=dev)
+    kern3r = timed_rotating([(lambda a=a, b=b, p=p: ops.matmul_reduce_scatter(a, b, p, rank, P, checksum=cs, out=out_r, workspace=ws3))
+                             for a, b, p in sets3])
+    del sets3
     sel = np.arange(0, rows, 61)
     _, want = oracle.matmul_reduce(A[sel].view(torch.int16).cpu().numpy().view(np.uint16), B.view(torch.int16).cpu().numpy().view(np.uint16),
                                    oracle.FP16, 0, len(sel), [p[sel].cpu().numpy() for p in peers])
     got = out[sel].view(torch.int16).cpu().numpy().view(np.uint16)
     rel = float(np.abs(got.view(np.float16).astype(np.float32) - want.view(np.float16).astype(np.float32)).max())
     res.append({"config": 3, "op": "matmul_reduce_scatter fp16 M=4096 K=1792 N=4096 P=8", "kernel_us": round(kern * 1e6, 2),
-                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * M * N * K / kern / 1e12, 1), "max_abs_err_sample": rel})
+                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * M * N * K / kern / 1e12, 1), "max_abs_err_sample": rel,
+                "kernel_us_rotating_inputs": round(kern3r * 1e6, 2), "input_sets_rotated": 4})
     # config 2: bf16 all-gather matmul, 8 shards [512,4096], B[4096,1024]
     m, K, N, P = 512, 4096, 1024, 8
     shards = [torch.randn((m, K), device=dev, generator=g).bfloat16() for _ in range(P)]
@@ -185,8 +208,14 @@ def float_configs(args, torch, L, ops, dev):
     out2 = torch.empty((m * P, N), dtype=torch.bfloat16, device=dev)
     ws2, f2 = slices(L.ALLGATHER_MATMUL, torch.bfloat16, m, K, N, 0, P)
     wall, kern = timed(lambda: ops.allgather_matmul(shards[0], shards[1:], B2, 0, P, out=out2, workspace=ws2))
+    sets2 = [(shards, B2)]
+    for _ in range(5):
+        sets2.append(([torch.randn((m, K), device=dev, generator=g).bfloat16() for _ in range(P)], (torch.randn((K, N), device=dev, generator=g) * 0.02).bfloat16()))
+    kern2r = timed_rotating([(lambda sh=sh, b=b: ops.allgather_matmul(sh[0], sh[1:], b, 0, P, out=out2, workspace=ws2)) for sh, b in sets2])
+    del sets2
     res.append({"config": 2, "op": "allgather_matmul bf16 8 x [512,4096] x [4096,1024]", "kernel_us": round(kern * 1e6, 2),
-                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * m * P * N * K / kern / 1e12, 1), "k_slices": f2})
+                "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * m * P * N * K / kern / 1e12, 1), "k_slices": f2,
+                "kernel_us_rotating_inputs": round(kern2r * 1e6, 2), "input_sets_rotated": 6})
     # config 1: fp16 all-reduce share, A[512,1024] (this rank's k half), B[1024,1024], one fp32 peer
     M, K, N, P = 512, 1024, 1024, 2
     A1 = (torch.rand((M, K), device=dev, generator=g) * 2 - 1).half()
@@ -202,7 +231,9 @@ def float_configs(args, torch, L, ops, dev):
         "metric": "fp16 matmul-reduce-scatter shard (BASELINE config 3) TFLOPS, 1 MI355X", "value": c3["TFLOPS"], "unit": "TFLOPS",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": c3["wall_us"] / 1e3, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
-        "config": {"workload": c3["op"] + ", 7 staged fp32 peers, fp16 [512,4096] kept"},
+        "config": {"workload": c3["op"] + ", 7 staged fp32 peers, fp16 [512,4096] kept",
+                   "note": "kernel_us: the same operands on every launch (88 MB for config 3, 42 MB for config 2: they stay in the Infinity Cache); "
+                           "kernel_us_rotating_inputs: another set of operands on every launch"},
         "roofline": {"bound": "mfma", "achieved": c3["TFLOPS"], "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(c3["TFLOPS"] / PEAK_F16_TFLOPS, 4), "traffic": None},
         "configs": res}))
