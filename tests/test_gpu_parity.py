@@ -773,6 +773,40 @@ def test_allgather_matmul_reads_shards_in_place(dtype, shape):
     _check_float(host16(out), want, full, dtype, K)
 
 
+@pytest.mark.parametrize("kslices", [False, True])
+def test_allgather_matmul_operands_streamed_from_hbm(kslices):
+    """All-gather matmul whose operands stream from HBM (four shards of [256, 8192] bf16 in separate allocations against
+    B [8192, 4096], 72 MB, 128 tiles): the six-stage ring with A copied in pairs of k steps out of the shard each tile row
+    belongs to, whole and in two k slices.  A sample of rows from every shard against the oracle, the rest of the output
+    through column sums against fp64."""
+    _need_gpu()
+    dtype = oracle.BF16
+    ml, N, K, P, rank = 256, 4096, 8192, 4, 1
+    g = torch.Generator(device=DEV).manual_seed(301)
+    dsh = [torch.randn((ml, K), device=DEV, generator=g).bfloat16() for _ in range(P)]     # P separate allocations
+    B = (torch.randn((K, N), device=DEV, generator=g) * 0.02).bfloat16()
+    ws = None
+    if kslices:
+        need, f = ops.kslice_plan(L.ALLGATHER_MATMUL, torch.bfloat16, ml, K, N, rank, P)
+        assert f == 2
+        ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    # the operator takes this rank's shard first, then the others in rank order: the gathered A is dsh in rank order
+    out = ops.allgather_matmul(dsh[rank], [dsh[r] for r in range(P) if r != rank], B, rank, P, workspace=ws)
+    torch.cuda.synchronize()
+    sel = np.arange(7, ml, 37)
+    shards_sel = [host16(d[sel]) for d in dsh]
+    want = oracle.allgather_matmul(shards_sel, host16(B), dtype)
+    full = oracle.gemm_half_f32(np.concatenate(shards_sel, 0), host16(B), dtype)
+    got = np.concatenate([host16(out[r * ml:(r + 1) * ml][sel]) for r in range(P)], 0)
+    _check_float(got, want, full, dtype, K)
+    a_all = torch.cat(dsh, 0).double()
+    col_sums = a_all.sum(0) @ B.double()                     # sum over all rows of every output column
+    got_sums = out.double().sum(0)
+    # every output element carries a bf16 rounding of at most 2^-9 relative
+    bound = (a_all.abs().sum(0) @ B.double().abs()) * 2.0 ** -8
+    assert bool(((got_sums - col_sums).abs() <= bound).all())
+
+
 @pytest.mark.parametrize("dtype", [oracle.BF16, oracle.FP16])
 def test_float_few_tiles_k_sliced(dtype):
     # two k slices per tile: an fp32 sum of two partials, the same whichever slice arrives last, so repeated
