@@ -122,7 +122,7 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     uint32_t m0 = t->m0, n0 = t->n0;
     if (n0 == 0) n0 = 256;
     const bool can256 = n0 == 256 && !transA && !transB && mRank % 256 == 0 && t->n % 256 == 0 &&
-                        ((uint64_t)t->k * es) % 128 == 0 && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
+                        ((uint64_t)t->k * es) % 128 == 0;
     if (m0 == 0) m0 = (mRank <= 64) ? 64 : 128;
     const bool dmaShape = can256 && m0 == 256;
     // (A as [k,m] exists in the 128-row direct-to-LDS kernel only: rows of m in whole 16-byte pieces, a rank's block on that grid)
@@ -138,7 +138,7 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     const bool ragged = plan.edge && m0 == 128 && mRank >= m0 && t->n >= n0 && ((uint64_t)t->k * es) % 64 == 0 && t->n % 8 == 0 &&
                         (transB || ((uint64_t)t->n * es) % 16 == 0);
     plan.dma = fastShape && (!plan.edge || ragged) && (m0 == 256 || (m0 == 128 && (!transB || ((uint64_t)t->k * es) % 16 == 0))) &&
-               (m0 == 128 || (!transA && !transB)) && !(d->flags & CATCOC_FLAG_REDUCE_INT32);
+               (m0 == 128 || (!transA && !transB));
     if (transA && !plan.dma) plan.variant = 0;   // the other fast kernels take A as [m,k] only
 
     GemmArgs &a = plan.args;
@@ -529,7 +529,7 @@ void launch_pipelined(bool quant, int dataType, void *computeStream, void *commS
         if (!check_ptr_align(p, a, b)) p.variant = 0;
     }
     g.nPeers = 0;
-    const bool dma = !quant && p.dma && !p.edge && p.variant != 0 && (uintptr_t)b % 16 == 0 && (g.ldb * 2) % 16 == 0 && (uintptr_t)d_out % 16 == 0;
+    const bool dma = p.dma && !p.edge && p.variant != 0 && (uintptr_t)b % 16 == 0 && (g.ldb * (quant ? 1 : 2)) % 16 == 0 && (uintptr_t)d_out % 16 == 0;
     g.flags &= ~(uint32_t)GF_RAGGED;   // (ragged problems run the bounds-checked kernel here)
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles and 16-byte aligned row-major operands"); return; }
     if (!dma && g.transA) p.variant = 0;
@@ -574,7 +574,8 @@ void launch_pipelined(bool quant, int dataType, void *computeStream, void *commS
         g.taskBase = first;
         g.taskCount = actual;
         if (he == hipSuccess)
-            e = dma ? (p.dtype == DT_F16 ? launch_gemm_dma_f16(g, computeStream) : launch_gemm_dma_bf16(g, computeStream))
+            e = dma ? (p.dtype == DT_I8 ? launch_gemm_dma_i8(g, computeStream)
+                       : p.dtype == DT_F16 ? launch_gemm_dma_f16(g, computeStream) : launch_gemm_dma_bf16(g, computeStream))
                     : launch_gemm(p.dtype, g, p.variant, p.edge, computeStream);
         if (e == 0 && he == hipSuccess) he = hipEventRecord(ready[r], cs);        // "store finished"
         if (e == 0 && he == hipSuccess) he = hipStreamWaitEvent(ms, ready[r], 0);

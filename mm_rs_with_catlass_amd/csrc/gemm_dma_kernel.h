@@ -895,11 +895,37 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
         }
     }
 
+    // W8A8 with GF_REDUCE_INT32 (the reference's data flow, quant_matmul_reduce_scatter.hpp:191-201,285-351): the peers'
+    // partials are int32 and join the accumulators before the dequantisation; tiles of other ranks leave as raw int32
+    // (explicit kept rows, RM, take fp32 partials only)
+    const bool redI32 = DT == DT_I8 && !RM && (args.flags & GF_REDUCE_INT32) != 0;
+    const uint32_t nPeersI32 = redI32 ? args.nPeers : 0u, nPeersF32 = redI32 ? 0u : args.nPeers;
     if (kept) {
         // (RM: a tile that starts above keptBegin makes this wrap; it is only added to rows of kept blocks, where the sum
         // is the row's index in the kept range again)
         const uint32_t out_row0 = ti.row - args.keptBegin;
         if constexpr (DT == DT_I8) {
+            // one int32 partial of the tile, 32 rows (64 loads per lane) at a time, as add_partial below does for fp32
+            for (uint32_t p = 0; p < nPeersI32; ++p) {
+                const int32_t *peer = (const int32_t *)args.peers[p] + args.peerRowOffset * args.peerLd;
+                const int32_t *src = peer + (int64_t)(int32_t)out_row0 * args.peerLd + (size_t)row_base * args.peerLd + gcol0;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const int32_t *srcb = src + (size_t)(mb * 32) * args.peerLd;
+                    int pv[16][4];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+#pragma unroll
+                        for (int nb = 0; nb < 4; ++nb)
+                            pv[r][nb] = __builtin_nontemporal_load(srcb + (size_t)((r >> 2) * 8 + (r & 3)) * args.peerLd + 32 * nb);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+#pragma unroll
+                        for (int nb = 0; nb < 4; ++nb) acc[mb][nb][r] += pv[r][nb];
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
             if (args.cAccum != nullptr) {
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
@@ -943,7 +969,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             constexpr int NBUF = 6;
             unsigned char *st = smem + w * 16384;
             __syncthreads();   // every wave has left the main loop's LDS reads behind
-            const uint32_t U = 2u * args.nPeers;   // units: peer u / 2, rows 16 (u & 1) .. of the block
+            const uint32_t U = 2u * nPeersF32;   // units: peer u / 2, rows 16 (u & 1) .. of the block
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
                 if constexpr (RM)
@@ -1041,7 +1067,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
-        for (uint32_t p = 0; p < args.nPeers; ++p) {
+        for (uint32_t p = 0; p < nPeersF32; ++p) {
             const float *peer = (const float *)args.peers[p] + args.peerRowOffset * args.peerLd;
             add_partial(peer + (int64_t)(int32_t)out_row0 * args.peerLd, args.peerLd, peer);
         }
@@ -1100,7 +1126,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                     float v;
                     if constexpr (DT == DT_I8) {
                         const int iv = acc[mb][nb][r];
-                        v = __fmul_rn(__fmul_rn((float)iv, sN[nb]), sM);
+                        v = redI32 ? i2f(iv) : __fmul_rn(__fmul_rn((float)iv, sN[nb]), sM);   // (raw int32: the bit pattern travels)
                     } else {
                         v = getf(mb, nb, r);
                     }

@@ -1161,6 +1161,74 @@ def test_quant_config4_full_size_properties():
     assert torch.equal(out0.view(torch.int16), want0.view(torch.int16))
 
 
+def test_quant_config4_full_size_int32_reduce():
+    """The reference's own W8A8 data flow at the benchmark size (M=8192, K=1792, N=4096, P=8): int32 peers join the
+    accumulators before the dequantisation (quant_matmul_reduce_scatter.hpp:285-351), the other ranks' tiles leave as raw
+    int32.  Exact integer checks of the whole kept block and of the workspace tiles, the output against the same fp32
+    products in torch, a row sample against the oracle, and the round-pipelined operator against the fused launch."""
+    _need_gpu()
+    import ctypes as C
+    M, N, K, P, rank = 8192, 4096, 1792, 8, 5
+    g = torch.Generator(device=DEV).manual_seed(44)
+    x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
+    x2 = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=DEV, generator=g)
+    s1 = torch.empty(M, device=DEV).uniform_(0.005, 0.02, generator=g)
+    s2 = torch.empty(N, device=DEV).uniform_(0.001, 0.01, generator=g)
+    bias = torch.randint(-1000, 1000, (N,), dtype=torch.int32, device=DEV, generator=g)
+    rows = M // P
+    peers = [torch.randint(-2 ** 24, 2 ** 24, (rows, N), dtype=torch.int32, device=DEV, generator=g) for _ in range(P - 1)]
+    # (one comm round holds all 1024 tasks: a single launch runs them in its own order, so no workspace stage may be reused)
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0, commInterval=4)
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    so = L.load()
+    need = so.catcoc_get_workspace_size(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, C.byref(t), C.byref(d))
+    ntasks = so.catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+    ob = torch.zeros(need // 4, dtype=torch.int32, device=DEV)
+    dump = torch.zeros((M, N), dtype=torch.int32, device=DEV)
+    cacc = torch.full((rows, N), -7, dtype=torch.int32, device=DEV)
+    out = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, bias, peers, rank, P, reduce_int32=True, acc_dump=dump, c_accum=cacc, outbound=ob,
+                                          tiling=t)
+    torch.cuda.synchronize()
+    # accumulators (bias included) through exact row sums; the kept block = accumulators + peers, exactly
+    want_rows = x1.double() @ x2.double().sum(1) + float(bias.to(torch.int64).sum())
+    assert torch.equal(dump.to(torch.int64).sum(1), want_rows.to(torch.int64))
+    kept = dump[rank * rows:(rank + 1) * rows].clone()
+    for p in peers:
+        kept += p
+    assert torch.equal(cacc, kept)
+    want = ((kept.float() * s2[None, :]) * s1[rank * rows:(rank + 1) * rows, None]).to(torch.bfloat16)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+    # row sample against the oracle, bit for bit
+    sel = np.arange(rank * rows, (rank + 1) * rows, 61)
+    acc_s, out_s = oracle.quant_matmul_reduce_scatter(
+        x1[sel].cpu().numpy(), x2.cpu().numpy(), s1[sel].cpu().numpy(), s2.cpu().numpy(), bias.cpu().numpy(), 0, len(sel),
+        [p[sel - rank * rows].cpu().numpy() for p in peers], oracle.BF16, reduce_int32=True)
+    assert np.array_equal(dump[sel].cpu().numpy(), acc_s)
+    assert np.array_equal(host16(out[sel - rank * rows]), out_s)
+    # raw int32 tiles of the other ranks where the reference puts them
+    obv = ob.view(-1, 256)
+    tr, row, col, ws = (C.c_uint32() for _ in range(4))
+    checked = 0
+    for task in range(0, ntasks, 7):
+        so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row), C.byref(col), C.byref(ws))
+        if tr.value == rank:
+            continue
+        assert torch.equal(obv[ws.value:ws.value + 128], dump[row.value:row.value + 128, col.value:col.value + 256]), task
+        checked += 1
+    assert checked > 100
+    # the round-pipelined operator (GEMM rounds and comm rounds on two streams) gives the same bits
+    del ob
+    t1 = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)   # four rounds of 256 tasks on two workspace stages
+    ob2 = _outbound_for(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, t1, rank, P, torch.int32)
+    side = torch.cuda.Stream()
+    for det in (True, False):
+        out2, cacc2 = ops.pipelined_quant_matmul_reduce_scatter(x1, x2, s1, s2, bias, peers, rank, P, ob2, tiling=t1, deterministic=det,
+                                                                comm_stream=side)
+        torch.cuda.synchronize()
+        assert torch.equal(cacc2, kept)
+        assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
+
+
 def test_float_config3_full_size_properties():
     """fp16 matmul-reduce-scatter benchmark config (A[4096,1792] N(0,1), B[1792,4096] N(0,0.02), P=8, 7 fp32 peers,
     kept block [512,4096]) at full size: 512 tiles of 128x256, the launch order of the many-tile regime.  A row sample
