@@ -10,8 +10,6 @@ in HBM before the timed region.  Prints ONE JSON line.
     python bench.py --mode copy     # plain 256 MiB device copy: the known-size kernel the HBM counters are scaled by
     python bench.py --mode decode   # BASELINE config 5: skinny-M sweep, K = N = 8192, GB/s per M (HBM-bound)
     python bench.py --mode float    # BASELINE configs 3 (fp16 reduce-scatter), 2 (bf16 all-gather) and 1 (fp16 all-reduce)
-    python bench.py --mode ceiling  # what the int8 matrix pipes sustain on this box without any memory traffic (power-limited)
-    python bench.py --mode probes   # the peer-partial stream on its own; LDS and direct-to-LDS copy rates of a CU
     python bench.py --mode sweep    # dynamic_tiling's sweep protocol on the MI355X-side knobs; writes the reference's result.csv
 """
 import argparse
@@ -25,6 +23,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
+# Which build of the dominant kernel profiles/traffic.json was recorded for; change both together whenever the kernel
+# or the launch routing of config 4 changes (the counter runs have to be repeated then).
+KERNEL_ID = "gemm_dma_kernel<int8,128x256,3 stages>+int32-reduce epilogue"
 
 
 def cpu_baseline(M, N, K, P, rank, repeats):
@@ -294,148 +295,12 @@ def tiling_sweep(args, torch, L, ops, dev):
         "best": best}))
 
 
-def mfma_ceiling(args, torch, L, dev):
-    """What the matrix pipes sustain on this box for the benchmark's operand distribution: the 128x256 kernel's inner loop
-    without any global-memory traffic (catcoc_probe_mfma_int8), with and without its LDS fragment reads, on uniform random
-    int8 (the benchmark's data) and on constant bytes."""
-    so = L.load()
-    g = torch.Generator(device=dev).manual_seed(20250101)
-    patterns = {"uniform int8 [-127,127]": torch.randint(-127, 128, (73728,), dtype=torch.int8, device=dev, generator=g),
-                "constant 1": torch.ones(73728, dtype=torch.int8, device=dev)}
-    sink = torch.zeros(512 * 256, dtype=torch.int32, device=dev)
-    steps = args.ceiling_steps
-    ops_per_launch = 512.0 * 4 * steps * 16 * 65536
-    res = []
-    for name, pat in patterns.items():
-        for lds in (1, 0):
-            def fn():
-                rc = so.catcoc_probe_mfma_int8(torch.cuda.current_stream().cuda_stream, lds, steps, pat.data_ptr(), sink.data_ptr())
-                assert rc == 0
-            for _ in range(args.warmup):
-                fn()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            e0.record()
-            for _ in range(args.steps):
-                fn()
-            e1.record()
-            torch.cuda.synchronize()
-            sec = e0.elapsed_time(e1) / 1e3 / args.steps
-            res.append({"data": name, "lds_fragment_reads": bool(lds), "ms_per_launch": round(sec * 1e3, 4),
-                        "TOPS": round(ops_per_launch / sec / 1e12, 1), "frac_of_peak": round(ops_per_launch / sec / 1e12 / PEAK_INT8_TOPS, 4)})
-    head = res[0]
-    print(json.dumps({
-        "metric": "int8 MFMA ceiling of the box: inner loop of the 128x256 kernel without global-memory traffic", "value": head["TOPS"],
-        "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_launch"],
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
-        "config": {"workload": "512 workgroups x 4 waves x %d k steps x 16 mfma_i32_32x32x32_i8; value = uniform random int8 with LDS reads" % steps},
-        "ceiling": res}))
-
-
-def memory_probes(args, torch, L, dev):
-    """Two measurement helpers behind the design notes: (1) the peer-partial stream of config 4 on its own (128 workgroups pull
-    seven [1024,4096] fp32 partials, rotating over four sets so that they come from HBM), in the accumulator layout of the
-    kept epilogue and in row layout with 16-byte loads at several depths; (2) what a CU's LDS and its direct-to-LDS copy path
-    deliver (bytes per second and per clock at the clock the device reports); (3) how much a workgroup that streams from HBM
-    or L2 slows the tile copies of the other workgroup on its CU."""
-    import ctypes as C
-    import numpy as np
-    so = L.load()
-    stream = lambda: torch.cuda.current_stream().cuda_stream
-    g = torch.Generator(device=dev).manual_seed(20250101)
-    rows, n, P, sets = 1024, 4096, 7, 4
-    bufs = [[torch.randn((rows, n), device=dev, generator=g) for _ in range(P)] for _ in range(sets)]
-    ptrs = [torch.tensor([b.data_ptr() for b in bs], dtype=torch.int64, device=dev) for bs in bufs]
-    sink = torch.zeros(512 * 256, dtype=torch.int32, device=dev)
-    nbytes = P * rows * n * 4
-
-    def timed(fn, reps):
-        for i in range(max(args.warmup, 2)):
-            fn(i)
-        ts = []
-        for i in range(reps):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            fn(i)
-            e1.record()
-            torch.cuda.synchronize()
-            ts.append(e0.elapsed_time(e1) * 1e-3)
-        return sum(ts) / len(ts), min(ts)
-
-    stream_res = []
-    evict = torch.zeros(1 << 27, dtype=torch.float32, device=dev)   # 512 MiB written between launches: nothing stays in the caches
-    for wrows in (128, rows):   # 16 workgroups (one tile row: far below what HBM delivers) and all 128
-        for name, layout, depth in (("accumulator layout, 64 four-byte loads per batch", 0, 0), ("row layout, 16-byte loads, 2 units in flight", 1, 2),
-                                    ("row layout, 3 units", 1, 3), ("row layout, 4 units", 1, 4), ("row layout, 6 units", 1, 6)):
-            def fn(i):
-                evict.add_(1.0)
-                rc = so.catcoc_probe_peer_stream(stream(), layout, depth, ptrs[i % sets].data_ptr(), P, wrows, n, sink.data_ptr())
-                assert rc == 0
-            ts = []
-            for i in range(max(args.steps, 20) + 2):
-                evict.add_(1.0)
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                rc = so.catcoc_probe_peer_stream(stream(), layout, depth, ptrs[i % sets].data_ptr(), P, wrows, n, sink.data_ptr())
-                e1.record()
-                torch.cuda.synchronize()
-                assert rc == 0
-                ts.append(e0.elapsed_time(e1) * 1e-3)
-            ts = ts[2:]
-            mean, best = sum(ts) / len(ts), min(ts)
-            wb = P * wrows * n * 4
-            stream_res.append({"workgroups": wrows // 128 * (n // 256), "variant": name, "us_mean": round(mean * 1e6, 1), "us_min": round(best * 1e6, 1),
-                               "TBps_mean": round(wb / mean / 1e12, 2), "GBps_per_workgroup_mean": round(wb / mean / 1e9 / (wrows // 128 * (n // 256)), 1)})
-    src = torch.randint(-127, 128, (32768,), dtype=torch.int8, device=dev, generator=g)
-    iters = 20000
-    cu, mhz = C.c_int(), C.c_int()
-    so.catcoc_device_info(C.byref(cu), C.byref(mhz), None, 0)
-    lds_res = []
-    for wgs in (256, 512):
-        for name, mode, rd, wr in (("16-byte LDS reads", 1, 8192, 0), ("transposing 8-byte LDS reads", 2, 8192, 0), ("both kinds of reads", 3, 16384, 0),
-                                   ("direct-to-LDS copies (source in the caches)", 4, 0, 6144), ("both reads and copies", 7, 16384, 6144)):
-            def fn(i):
-                rc = so.catcoc_probe_lds(stream(), mode, wgs, iters, src.data_ptr(), sink.data_ptr())
-                assert rc == 0
-            mean, best = timed(fn, 5)
-            per_cu = (rd + wr) * 4.0 * iters * (wgs / float(cu.value))
-            lds_res.append({"what": name, "workgroups_per_cu": wgs // 256, "ms_min": round(best * 1e3, 3), "GBps_per_cu": round(per_cu / best / 1e9, 1),
-                            "bytes_per_clock_per_cu_at_%d_MHz" % mhz.value: round(per_cu / best / (mhz.value * 1e6), 1),
-                            "read_share": round(rd / float(rd + wr), 2)})
-    # (3) a streaming neighbour on the CU
-    hot = torch.randint(-127, 128, (256 * 98304 + 256 * 65536,), dtype=torch.int8, device=dev, generator=g)
-    big = torch.zeros(1 << 28, dtype=torch.float32, device=dev)
-    ticks = torch.zeros(256, dtype=torch.int64, device=dev)
-    hwid = torch.zeros(512, dtype=torch.int32, device=dev)
-    nsteps = 200
-    nb_res = []
-    for rep in range(2):
-        for mode, name in ((0, "the CU's other workgroup exits at once"), (1, "it streams from HBM (batches of 64 four-byte loads, awaited)"),
-                           (2, "it streams the same way from L2")):
-            rc = so.catcoc_probe_neighbour(stream(), mode, nsteps, hot.data_ptr(), big.data_ptr(), sink.data_ptr(), ticks.data_ptr(), hwid.data_ptr())
-            assert rc == 0
-            torch.cuda.synchronize()
-            t = ticks.cpu().numpy() / 100.0   # us
-            h = hwid.cpu().numpy()
-            if rep == 1:
-                nb_res.append({"neighbour": name, "us_per_copy_step_median": round(float(np.median(t)) / nsteps, 3),
-                               "us_per_copy_step_max": round(float(t.max()) / nsteps, 3),
-                               "pairs_w_and_w_plus_256_on_one_cu": int((h[:256] == h[256:]).sum())})
-    head = [r for r in stream_res if r["workgroups"] == 128][0]
-    print(json.dumps({
-        "metric": "peer-partial stream of config 4 on its own (7 x [1024,4096] fp32, 128 workgroups), accumulator layout", "value": head["TBps_mean"],
-        "unit": "TB/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": max(args.warmup, 2), "ms_per_step": head["us_mean"] / 1e3,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "measurement helpers: catcoc_probe_peer_stream and catcoc_probe_lds"},
-        "peer_stream": stream_res, "lds_and_copy_path": lds_res, "streaming_neighbour": nb_res}))
-
-
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode", "float", "sweep", "ceiling", "probes"], default="kept",
+    ap.add_argument("--mode", choices=["kept", "outbound", "copy", "decode", "float", "sweep"], default="kept",
                     help="kept: non-kept tiles are folded into checksums (BASELINE's literal outputs); "
                          "outbound: they are also stored as fp32 to the symmetric workspace")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -445,7 +310,6 @@ def main():
     ap.add_argument("--sets", type=int, default=4, help="independent input sets the launches rotate over (1 = same buffers every launch)")
     ap.add_argument("--sustained", type=int, default=300, help="launches of the untimed sustained block (0 = skip)")
     ap.add_argument("--no-other-mode", action="store_true", help="skip the secondary run of the other store mode")
-    ap.add_argument("--ceiling-steps", type=int, default=20000, help="--mode ceiling: k steps per launch of the probe")
     ap.add_argument("--csv", default="", help="--mode sweep: where result.csv goes (default: result.csv in the working directory)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -485,12 +349,6 @@ def main():
         return
     if args.mode == "sweep":
         tiling_sweep(args, torch, L, ops, dev)
-        return
-    if args.mode == "probes":
-        memory_probes(args, torch, L, dev)
-        return
-    if args.mode == "ceiling":
-        mfma_ceiling(args, torch, L, dev)
         return
     M, K, N, P, rank = 8192, 1792, 4096, 8, args.rank
     rows = M // P
@@ -632,11 +490,17 @@ def main():
     value = ops_per_step / wall_s / 1e12
     achieved = ops_per_step / avg_kernel_s / 1e12
     info = ops.device_info()
+    # HBM bytes per launch come from two counter runs under rocprofv3 (FETCH_SIZE, WRITE_SIZE), not from this run: the
+    # figure recorded for this kernel and mode is quoted with its source, or null when the record names another kernel
     traffic = None
+    traffic_source = None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get("quant_rs_config4_" + args.mode)
+            rec = json.load(open(tpath))
+            if rec.get("kernel") == KERNEL_ID and args.m0 == 0:
+                traffic = rec.get("quant_rs_config4_" + args.mode)
+                traffic_source = "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, recorded for kernel id '%s'); not measured in this run" % KERNEL_ID
         except Exception:
             traffic = None
     sustained_s = sum(series[5:]) / len(series[5:]) if series else None
@@ -650,7 +514,7 @@ def main():
                    "mode": args.mode, "tile": "%dx256x64" % (tiling.m0 or 128), "tasks": int(ntasks),
                    "input_sets_rotated": len(sets), "parity_sample_ok": parity_ok},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                     "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": traffic,
+                     "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "kernel_us_avg": round(avg_kernel_s * 1e6, 2),
                      "kernel_us_avg_same_buffers": round(hot_kernel_s * 1e6, 2),
                      "kernel_us_sustained": round(sustained_s * 1e6, 2) if sustained_s else None,

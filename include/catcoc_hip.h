@@ -113,6 +113,7 @@ typedef void (*CatcocKernelFuncPtr)(void *stream, uint64_t fftsAddr, uint8_t *a,
  * (examples/dynamic_tiling/impl/kernel/matmul_reduce_scatter.h:155-156): which
  * rank this GPU plays and where the other ranks' staged data live.  Zero-filled
  * fields take the documented defaults. */
+struct CatcocPipelinedPlan;
 typedef struct CatcocSymmetricDesc {
     uint32_t magic;           /* CATCOC_DESC_MAGIC */
     uint32_t rankIdx;         /* shmem_my_pe() */
@@ -150,6 +151,10 @@ typedef struct CatcocSymmetricDesc {
      * stream, or ordered by events). */
     void *workspace;
     uint64_t workspaceBytes;
+    /* Round-pipelined operators only: the events they order their two streams with, made once by
+     * catcoc_pipelined_plan_create and reused by every call that is given the plan (NULL = the call makes and destroys
+     * its own).  Calls that share a plan must not overlap. */
+    struct CatcocPipelinedPlan *pipelinedPlan;
 } CatcocSymmetricDesc;
 
 /* ----------------------------------------------------------------------- */
@@ -208,8 +213,8 @@ CATCOC_API void catcoc_launch_quant_matmul_reduce_scatter(void *stream, uint64_t
  * until the process ends.  The call allocates nothing.  A launch that needs more scratch than that is rejected
  * (catcoc_last_error() says how much it needs).  All calls on one GPU share that GPU's array: calls that overlap on
  * one GPU (different streams, no ordering between them) race; calls on one stream, or ordered by events, are fine.
- * The first call on a GPU also queues a small kernel on `stream` that zeroes the array's counter block; afterwards
- * every launch leaves the counters at zero for the next. */
+ * Nothing is cleared at run time: the array is zero when the library's code is loaded on a GPU, and every launch leaves
+ * its counter block at zero again for the next, also when it is replayed from a HIP graph. */
 #define CATCOC_STATIC_SCRATCH_BYTES (CATCOC_WORKSPACE_COUNTER_BYTES + (32u << 20))
 CATCOC_API void catcoc_launch_quant_matmul_reduce_scatter_static_scratch(void *stream, uint64_t fftsAddr, uint8_t *x1,
     uint8_t *x2, uint8_t *scale_x1, uint8_t *scale_x2, uint8_t *bias, uint8_t *c_accum, uint8_t *d_out,
@@ -225,7 +230,8 @@ CATCOC_API void catcoc_launch_quant_matmul_reduce_scatter_static_scratch(void *s
  * the kept rank's into the local block, the others into stage `round % workspaceStages` of desc->outbound in the
  * tile-linear layout -- then the comm side (on commStream) adds the peers' blocks into the local block along
  * BlockCommSwizzle's task list; the GEMM of round + workspaceStages waits for that before it reuses the stage.  The two
- * cross-core flags per stage are HIP events between the two streams (created and destroyed inside the call); on return
+ * cross-core flags per stage are HIP events between the two streams (created and destroyed inside the call unless the
+ * descriptor names a CatcocPipelinedPlan, below); on return
  * computeStream is ordered after the finished output.  commBlockM (0 = 64) must divide m0; commDataSplit x commNpuSplit
  * is the number of comm "cores" (workgroups), raised to 256 x 1 when below 16.
  *   W8A8: int32 tiles; peers[] are int32 partials [m/P, n] added into c_accum (required, receives the reduced int32
@@ -244,6 +250,20 @@ CATCOC_API void catcoc_pipelined_quant_matmul_reduce_scatter(void *computeStream
 CATCOC_API void catcoc_pipelined_matmul_reduce_scatter(void *computeStream, void *commStream, int dataType, uint8_t *a,
     uint8_t *b, uint8_t *c, uint8_t *symmetricPtr, CocTilingParams *tiling, uint32_t transA, uint32_t transB,
     uint32_t deterministic);
+
+/* The events of the round-pipelined operators as an object of the caller's.  The reference needs nothing of the kind:
+ * its two flags per workspace stage live in the symmetric workspace and the one kernel waits on them itself
+ * (quant_matmul_reduce_scatter.hpp:159-164,219,282,319); here they are HIP events between two streams, and a call that
+ * has to create them cannot run under stream capture or in a loop that must not allocate.  A plan holds the events for
+ * calls of up to maxRounds comm rounds (catcoc_pipelined_round_count says how many a call has) on the device that is
+ * current when it is made; a call whose descriptor names the plan creates and destroys nothing, so it can be captured
+ * into a HIP graph (capture on computeStream; commStream joins the capture through the first event and is joined back
+ * before the call returns).  catcoc_pipelined_plan_create returns NULL on failure (catcoc_last_error() says why). */
+typedef struct CatcocPipelinedPlan CatcocPipelinedPlan;
+CATCOC_API CatcocPipelinedPlan *catcoc_pipelined_plan_create(uint32_t maxRounds);
+CATCOC_API void catcoc_pipelined_plan_destroy(CatcocPipelinedPlan *plan);
+/* Comm rounds of a round-pipelined call with this tiling and descriptor: ceil(tasks / (blockNum * commInterval)); 0 on error. */
+CATCOC_API uint32_t catcoc_pipelined_round_count(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc);
 
 /* SplitkMatmul's ReduceAdd as a kernel of its own (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:24-161):
  * src holds splitkFactor fp32 slices of elementCount elements each, back to back; dst[i] = the slices' sum in slice order
@@ -394,37 +414,6 @@ CATCOC_API int catcoc_launch_tile(int commType, const CocTilingParams *tiling, c
 /* The task workgroup `wg` of a launch with `tasks` tasks runs (XCD-aware chunking unless
  * CATCOC_FLAG_LINEAR_ORDER); a bijection on [0,tasks). */
 CATCOC_API uint32_t catcoc_workgroup_task(uint32_t wg, uint32_t tasks, uint32_t flags);
-
-/* Measurement helper (no counterpart in the reference): the 128x256 W8A8 kernel's inner loop without its global-memory
- * side -- 512 workgroups of four waves, sixteen 32x32x32 int8 MFMAs per wave and step, with (ldsReads != 0) or without
- * the LDS fragment reads that feed them -- on the 73728 bytes at `pattern` (device memory, 16-byte aligned), which every
- * workgroup copies into its LDS first.  sink: 512 * 256 * 4 bytes of device memory.  Ops of a launch:
- * 512 * 4 * steps * 16 * 65536.  It measures what the matrix pipes sustain for that data on the box at hand (they are
- * power-limited); bench.py --mode ceiling reports it next to the operator's rate.  Returns 0 on success. */
-CATCOC_API int catcoc_probe_mfma_int8(void *stream, uint32_t ldsReads, uint32_t steps, const uint8_t *pattern, uint8_t *sink);
-/* Measurement helper (no counterpart in the reference): the peer-partial stream of a reduce-scatter launch on its own.  One
- * workgroup per 128x256 tile of a [rows, n] fp32 block (row pitch n; rows % 128 == 0, n % 256 == 0) adds up the nPeers
- * partials at peers[] (a DEVICE array of device pointers).  layout 0: accumulator layout, 64 four-byte loads per lane, peer
- * and 32-row block, awaited before they are added (the kept epilogue of the 128-row kernel); layout 1: row layout, sixteen-byte
- * loads in units of eight with `depth` (2, 3, 4 or 6) units in flight (the pipelined epilogue; nPeers must be 7).
- * sink: tiles * 256 * 4 bytes.  Returns 0 on success. */
-CATCOC_API int catcoc_probe_peer_stream(void *stream, uint32_t layout, uint32_t depth, const void *const *peers, uint32_t nPeers,
-                                        uint32_t rows, uint32_t n, uint8_t *sink);
-/* Measurement helper (no counterpart in the reference): LDS read and direct-to-LDS copy rates of a CU.  `workgroups` (256 = one
- * per CU, 512 = two) workgroups of four waves with 72 KiB of LDS run `iters` iterations; per iteration and wave, by mode bit:
- * 1 = eight 16-byte LDS reads (8 KiB), 2 = sixteen transposing 8-byte LDS reads (8 KiB), 4 = six 1 KiB direct-to-LDS copies from
- * the 24 KiB at `src` (device memory, 16-byte aligned; it stays in the caches).  Modes 1, 2, 3, 4, 7.  sink: workgroups * 256 * 4
- * bytes.  Returns 0 on success. */
-CATCOC_API int catcoc_probe_lds(void *stream, uint32_t mode, uint32_t workgroups, uint32_t iters, const uint8_t *src, uint8_t *sink);
-/* Measurement helper (no counterpart in the reference): what a streaming workgroup costs the other workgroup on its CU.  512
- * workgroups, two per CU (w and w + 256).  The first 256 run the copy side of a main loop -- per step six 1 KiB direct-to-LDS
- * copies per wave, two steps ahead, from 96 KiB of their own inside `hot` (device memory, 256 * 98304 + 256 * 65536 bytes,
- * 16-byte aligned) -- for `steps` steps and leave their duration in ticks[w] (100 MHz ticks).  The other 256 exit at once
- * (mode 0), or fetch steps / 2 batches of 64 four-byte loads per lane, each batch awaited, from 4 MiB of their own inside `big`
- * (1 GiB of device memory; mode 1) or from 64 KiB of their own at the end of `hot` (mode 2).  hwid[w], w < 512: bits 0-7 CU /
- * shader array / shader engine of the workgroup, bits 8.. its XCD.  sink: 256 * 256 * 4 bytes.  Returns 0 on success. */
-CATCOC_API int catcoc_probe_neighbour(void *stream, uint32_t mode, uint32_t steps, const uint8_t *hot, const uint8_t *big, uint8_t *sink,
-                                      uint64_t *ticks, uint32_t *hwid);
 
 /* Library / device information: fills cuCount, clockMHz of the current device; returns 0 on success. */
 CATCOC_API int catcoc_device_info(int *cuCount, int *clockMHz, char *name, int nameLen);

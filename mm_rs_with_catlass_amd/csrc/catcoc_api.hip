@@ -9,6 +9,7 @@
 
 #include <math.h>
 
+#include <new>
 #include <vector>
 
 #include "catcoc_hip.h"
@@ -407,6 +408,13 @@ void launch_quant_splitk(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_
         return;
     }
     GemmArgs &a = sp.args;
+    // The large-tile route picked its k slices by itself (no desc.splitK): they need a workspace to meet through, and without
+    // one that fits the tiles run whole, as any other few-tile launch of that kernel does.  Only an explicit splitK insists.
+    if (sp.large && sp.f > 1 && d->splitK == 0 &&
+        (d->workspace == nullptr || (uintptr_t)d->workspace % 256 != 0 || d->workspaceBytes < sp.workspaceBytes)) {
+        sp.f = 1;
+        a.splitK = 0;
+    }
     if (sp.f > 1) {
         if (d->workspace == nullptr || d->workspaceBytes < sp.workspaceBytes) {
             fail(E_WORKSPACE, "split factor %u needs a zero-initialised workspace of %llu bytes (catcoc_get_splitk_workspace_size)",
@@ -471,6 +479,48 @@ void launch_quant(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_x1, uin
     const int e = dma ? launch_gemm_dma_i8(p.args, stream) : launch_gemm(p.dtype, p.args, p.variant, p.edge, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
     ok();
+}
+
+}  // namespace
+
+// The events of a round-pipelined call: "store finished" and "compute finished" per round, and the join at the end.
+struct CatcocPipelinedPlan {
+    uint32_t magic = 0;
+    std::vector<hipEvent_t> ready, done;
+    hipEvent_t fin = nullptr;
+};
+
+namespace {
+
+constexpr uint32_t kPlanMagic = 0x4350504cu;   // "CPPL"
+
+void plan_destroy_events(CatcocPipelinedPlan &p)
+{
+    for (hipEvent_t e : p.ready) if (e) (void)hipEventDestroy(e);
+    for (hipEvent_t e : p.done) if (e) (void)hipEventDestroy(e);
+    if (p.fin) (void)hipEventDestroy(p.fin);
+    p.ready.clear();
+    p.done.clear();
+    p.fin = nullptr;
+    p.magic = 0;
+}
+
+bool plan_make_events(CatcocPipelinedPlan &p, uint32_t rounds)
+{
+    p.ready.assign(rounds, nullptr);
+    p.done.assign(rounds, nullptr);
+    hipError_t he = hipEventCreateWithFlags(&p.fin, hipEventDisableTiming);
+    for (uint32_t r = 0; r < rounds && he == hipSuccess; ++r) {
+        he = hipEventCreateWithFlags(&p.ready[r], hipEventDisableTiming);
+        if (he == hipSuccess) he = hipEventCreateWithFlags(&p.done[r], hipEventDisableTiming);
+    }
+    if (he != hipSuccess) {
+        plan_destroy_events(p);
+        fail(E_LAUNCH, "hipEventCreate failed: %s", hipGetErrorString(he));
+        return false;
+    }
+    p.magic = kPlanMagic;
+    return true;
 }
 
 // ---- round-pipelined, reference-faithful form of the reduce-scatter operators ------------------
@@ -552,20 +602,23 @@ void launch_pipelined(bool quant, int dataType, void *computeStream, void *commS
 
     const uint32_t bpc = sp.blockPerComm, perRank = bpc / P, stages = sp.stages;
     const uint32_t rounds = ceil_div(sp.coreLoops, bpc);
-    std::vector<hipEvent_t> ready(rounds), done(rounds);
-    hipEvent_t fin = nullptr;
-    auto destroy = [&]() {
-        for (hipEvent_t e : ready) if (e) (void)hipEventDestroy(e);
-        for (hipEvent_t e : done) if (e) (void)hipEventDestroy(e);
-        if (fin) (void)hipEventDestroy(fin);
-    };
-    for (uint32_t r = 0; r < rounds; ++r) ready[r] = done[r] = nullptr;
-    hipError_t he = hipEventCreateWithFlags(&fin, hipEventDisableTiming);
-    for (uint32_t r = 0; r < rounds && he == hipSuccess; ++r) {
-        he = hipEventCreateWithFlags(&ready[r], hipEventDisableTiming);
-        if (he == hipSuccess) he = hipEventCreateWithFlags(&done[r], hipEventDisableTiming);
+    // the events: the caller's plan, or a set made for this call alone
+    CatcocPipelinedPlan own;
+    CatcocPipelinedPlan *plan = given->pipelinedPlan;
+    if (plan != nullptr) {
+        if (plan->magic != kPlanMagic) { fail(E_DESC, "desc.pipelinedPlan does not point at a CatcocPipelinedPlan"); return; }
+        if (plan->ready.size() < rounds) {
+            fail(E_WORKSPACE, "this call has %u comm rounds; the plan holds events for %u", rounds, (uint32_t)plan->ready.size());
+            return;
+        }
+    } else {
+        plan = &own;
+        if (!plan_make_events(own, rounds)) return;
     }
-    if (he != hipSuccess) { destroy(); fail(E_LAUNCH, "hipEventCreate failed: %s", hipGetErrorString(he)); return; }
+    std::vector<hipEvent_t> &ready = plan->ready, &done = plan->done;
+    hipEvent_t fin = plan->fin;
+    auto destroy = [&]() { if (plan == &own) plan_destroy_events(own); };
+    hipError_t he = hipSuccess;
     hipStream_t cs = (hipStream_t)computeStream, ms = (hipStream_t)commStream;
     int e = 0;
     for (uint32_t r = 0; r < rounds && e == 0 && he == hipSuccess; ++r) {
@@ -601,19 +654,14 @@ void launch_pipelined(bool quant, int dataType, void *computeStream, void *commS
 // needs the memory (kernel arguments, the fill below) uses the per-device address obtained from it.
 static __device__ __align__(256) unsigned char scratch[CATCOC_STATIC_SCRATCH_BYTES];
 
-__global__ void scratch_zero_kernel(uint32_t *p, uint32_t words)
-{
-    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x) p[i] = 0u;
-}
-
 constexpr int kMaxDevices = 64;
-struct ScratchState { void *ptr; bool cleared; };
+struct ScratchState { void *ptr; };
 ScratchState g_scratch[kMaxDevices];
 pthread_mutex_t g_scratchLock = PTHREAD_MUTEX_INITIALIZER;
 
-// Address of the current device's copy of `scratch`; on the first call on a device also queues, on `stream`, a kernel
-// that zeroes the counter block (a kernel, not a memset: the call may be under stream capture).  NULL on failure.
-void *scratch_for_current_device(void *stream)
+// Address of the current device's copy of `scratch`; NULL on failure.  Nothing has to be cleared: a __device__ array is
+// zero when the code object is loaded, and every launch leaves the counter block at zero again for the next.
+void *scratch_for_current_device()
 {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
@@ -631,17 +679,6 @@ void *scratch_for_current_device(void *stream)
             return nullptr;
         }
         st.ptr = p;
-    }
-    if (!st.cleared) {
-        hipLaunchKernelGGL(scratch_zero_kernel, dim3(16), dim3(256), 0, (hipStream_t)stream, (uint32_t *)st.ptr,
-                           (uint32_t)(kCounterBlockBytes / 4u));
-        const hipError_t e = hipGetLastError();
-        if (e != hipSuccess) {
-            pthread_mutex_unlock(&g_scratchLock);
-            fail(E_LAUNCH, "clearing the built-in scratch failed: %s", hipGetErrorString(e));
-            return nullptr;
-        }
-        st.cleared = true;
     }
     void *p = st.ptr;
     pthread_mutex_unlock(&g_scratchLock);
@@ -690,7 +727,7 @@ void catcoc_launch_quant_matmul_reduce_scatter_static_scratch(void *stream, uint
         return;
     }
     if (need != 0) {
-        void *p = scratch_for_current_device(stream);
+        void *p = scratch_for_current_device();
         if (p == nullptr) return;
         d.workspace = p;
         d.workspaceBytes = CATCOC_STATIC_SCRATCH_BYTES;
@@ -1083,6 +1120,41 @@ void catcoc_pipelined_quant_matmul_reduce_scatter(void *computeStream, void *com
     (void)fftsAddr;
     launch_pipelined(true, INT8, computeStream, commStream, x1, x2, scale_x1, scale_x2, bias, c_accum, d_out, symmetricPtr, tiling, transA,
                      transB, outDataType, deterministic);
+}
+
+CatcocPipelinedPlan *catcoc_pipelined_plan_create(uint32_t maxRounds)
+{
+    if (maxRounds == 0 || maxRounds > 65536u) { fail(E_TILING, "maxRounds %u out of range 1..65536", maxRounds); return nullptr; }
+    CatcocPipelinedPlan *p = new (std::nothrow) CatcocPipelinedPlan();
+    if (p == nullptr) { fail(E_LAUNCH, "out of host memory"); return nullptr; }
+    if (!plan_make_events(*p, maxRounds)) { delete p; return nullptr; }
+    ok();
+    return p;
+}
+
+void catcoc_pipelined_plan_destroy(CatcocPipelinedPlan *plan)
+{
+    if (plan == nullptr) return;
+    plan_destroy_events(*plan);
+    delete plan;
+}
+
+uint32_t catcoc_pipelined_round_count(int commType, const CocTilingParams *tiling, const CatcocSymmetricDesc *desc)
+{
+    if (desc == nullptr || desc->magic != CATCOC_DESC_MAGIC) { fail(E_DESC, "desc does not point at a CatcocSymmetricDesc"); return 0; }
+    if (commType != MATMUL_REDUCE_SCATTER && commType != QUANT_MATMUL_REDUCE_SCATTER) {
+        fail(E_DTYPE, "the round-pipelined form exists for the reduce-scatter operators (commType %d)", commType);
+        return 0;
+    }
+    CatcocSymmetricDesc q = *desc;
+    for (int i = 0; i < CATCOC_MAX_RANKS; ++i) if (!q.peers[i]) q.peers[i] = (const void *)16;
+    q.flags &= ~CATCOC_OUTBOUND_MASK;
+    q.workspace = nullptr;
+    q.splitK = 0;
+    Plan p;
+    if (make_plan(commType, commType == QUANT_MATMUL_REDUCE_SCATTER ? INT8 : FP16, tiling, &q, 0, 0, p)) return 0;
+    ok();
+    return ceil_div(p.args.sched.coreLoops, p.args.sched.blockPerComm);
 }
 
 void catcoc_pipelined_matmul_reduce_scatter(void *computeStream, void *commStream, int dataType, uint8_t *a, uint8_t *b, uint8_t *c,

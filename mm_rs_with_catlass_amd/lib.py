@@ -48,6 +48,7 @@ class CatcocSymmetricDesc(C.Structure):
         ("outbound", C.c_void_p), ("outboundBytes", C.c_uint64),
         ("checksum", C.c_void_p), ("accDump", C.c_void_p),
         ("workspace", C.c_void_p), ("workspaceBytes", C.c_uint64),
+        ("pipelinedPlan", C.c_void_p),
     ]
 
 
@@ -74,7 +75,7 @@ EXPORTS = [
     "catcoc_device_info", "catcoc_version",
     "catcoc_pipelined_quant_matmul_reduce_scatter", "catcoc_pipelined_matmul_reduce_scatter", "catcoc_reduce_add",
     "catcoc_verify", "catcoc_comm_block_idx_ex", "catcoc_comm_core_loop", "catcoc_task_tiles",
-    "catcoc_probe_mfma_int8", "catcoc_probe_peer_stream", "catcoc_probe_lds", "catcoc_probe_neighbour",
+    "catcoc_pipelined_plan_create", "catcoc_pipelined_plan_destroy", "catcoc_pipelined_round_count",
 ]
 
 _lib = None
@@ -189,14 +190,12 @@ def load():
     L.catcoc_comm_core_loop.restype = u32
     L.catcoc_task_tiles.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc), u32, u32] + [pu] * 4
     L.catcoc_task_tiles.restype = u32
-    L.catcoc_probe_mfma_int8.argtypes = [vp, u32, u32, vp, vp]
-    L.catcoc_probe_mfma_int8.restype = C.c_int
-    L.catcoc_probe_peer_stream.argtypes = [vp, u32, u32, vp, u32, u32, u32, vp]
-    L.catcoc_probe_peer_stream.restype = C.c_int
-    L.catcoc_probe_lds.argtypes = [vp, u32, u32, u32, vp, vp]
-    L.catcoc_probe_lds.restype = C.c_int
-    L.catcoc_probe_neighbour.argtypes = [vp, u32, u32, vp, vp, vp, vp, vp]
-    L.catcoc_probe_neighbour.restype = C.c_int
+    L.catcoc_pipelined_plan_create.argtypes = [u32]
+    L.catcoc_pipelined_plan_create.restype = vp
+    L.catcoc_pipelined_plan_destroy.argtypes = [vp]
+    L.catcoc_pipelined_plan_destroy.restype = None
+    L.catcoc_pipelined_round_count.argtypes = [C.c_int, C.POINTER(CocTilingParams), C.POINTER(CatcocSymmetricDesc)]
+    L.catcoc_pipelined_round_count.restype = u32
     _lib = L
     return L
 

@@ -331,9 +331,39 @@ def allgather_matmul(a_local, peer_shards, b, rank=0, rank_size=1, tiling=None, 
                      workspace, split_k)
 
 
+class PipelinedPlan:
+    """The events of the round-pipelined operators, made once (catcoc_pipelined_plan_create) and reused by every call
+    that is given the plan: such a call creates nothing and can be captured into a HIP graph."""
+
+    def __init__(self, max_rounds):
+        self.handle = _l.load().catcoc_pipelined_plan_create(int(max_rounds))
+        if not self.handle:
+            raise _l.CatcocError(_l.last_error())
+        self.max_rounds = int(max_rounds)
+
+    def close(self):
+        if self.handle:
+            _l.load().catcoc_pipelined_plan_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def pipelined_round_count(comm_type, tiling, rank, rank_size, block_num=0, stages=0):
+    """Comm rounds a round-pipelined call with this tiling has (catcoc_pipelined_round_count)."""
+    d = _l.make_desc(rank, rank_size, [16] * (rank_size - 1), block_num=block_num, stages=stages)
+    n = _l.load().catcoc_pipelined_round_count(comm_type, C.byref(tiling), C.byref(d))
+    _l.check()
+    return n
+
+
 def pipelined_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias, peers, rank, rank_size, outbound, c_accum=None,
                                           out_dtype=torch.bfloat16, tiling=None, trans_b=False, peer_row_offset=0, deterministic=True,
-                                          comm_stream=None, block_num=0, stages=0, swizzle=None, out=None):
+                                          comm_stream=None, block_num=0, stages=0, swizzle=None, out=None, plan=None):
     """The W8A8 operator in the reference's round-pipelined form (catcoc_pipelined_quant_matmul_reduce_scatter): GEMM rounds
     on torch's current stream, comm rounds (int32 peers added into c_accum) and the dequant pass on comm_stream.
     peers: rank_size-1 int32 partials [m/rank_size, n]; outbound: the symmetric workspace (bytes per
@@ -362,6 +392,8 @@ def pipelined_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias, peer
     _check_dev(x1, x2, scale_x1, scale_x2, bias, outbound, c_accum, out, *peers)
     t = tiling if tiling is not None else default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, 0, block_num, stages, swizzle, outbound, None, None)
+    if plan is not None:
+        d.pipelinedPlan = plan.handle
     cs = comm_stream if comm_stream is not None else torch.cuda.current_stream()
     _l.load().catcoc_pipelined_quant_matmul_reduce_scatter(
         _stream(), cs.cuda_stream, 0, x1.data_ptr(), x2.data_ptr(), scale_x1.data_ptr(), scale_x2.data_ptr(), _ptr(bias),
@@ -372,7 +404,7 @@ def pipelined_quant_matmul_reduce_scatter(x1, x2, scale_x1, scale_x2, bias, peer
 
 def pipelined_matmul_reduce_scatter(a, b, peers, rank, rank_size, outbound, tiling=None, trans_a=False, trans_b=False,
                                     peer_row_offset=0, deterministic=True, comm_stream=None, block_num=0, stages=0, swizzle=None,
-                                    out=None, acc_dump=None):
+                                    out=None, acc_dump=None, plan=None):
     """fp16 / bf16 reduce-scatter in the reference's round-pipelined form and precision: the local partial is rounded to the
     16-bit type, peers are 16-bit partials [m/rank_size, n] of the same type, every add rounds to that type."""
     if a.dtype not in _TORCH_TO_DT or b.dtype != a.dtype:
@@ -397,6 +429,8 @@ def pipelined_matmul_reduce_scatter(a, b, peers, rank, rank_size, outbound, tili
     _check_dev(a, b, outbound, out, acc_dump, *peers)
     t = tiling if tiling is not None else default_tiling(m, k, n, rank_size, m0=0, n0=0, k0=0)
     d = _desc(rank, rank_size, list(peers), peer_row_offset, 0, block_num, stages, swizzle, outbound, None, acc_dump)
+    if plan is not None:
+        d.pipelinedPlan = plan.handle
     cs = comm_stream if comm_stream is not None else torch.cuda.current_stream()
     _l.load().catcoc_pipelined_matmul_reduce_scatter(_stream(), cs.cuda_stream, _TORCH_TO_DT[a.dtype], a.data_ptr(), b.data_ptr(),
                                                      out.data_ptr(), C.addressof(d), C.byref(t), int(trans_a), int(trans_b), int(deterministic))

@@ -67,6 +67,56 @@ def test_static_scratch_entry_point_matches_the_allocating_one():
         want, got = _both(so, x1, x2, s1, s2, bias, peers, t, d_ws, d_static)
         assert not torch.isnan(want.float()).any()
         assert torch.equal(want.view(torch.int16), got.view(torch.int16)), (M, K, N, P, kr)
+        if kr is not None:       # the skinny cases are small enough for the CPU oracle: bit for bit against it as well
+            import oracle
+            _, out_want = oracle.quant_matmul_reduce_scatter(
+                x1.cpu().numpy(), x2.cpu().numpy(), s1.cpu().numpy(), s2.cpu().numpy(), bias.cpu().numpy(), 0, kr,
+                [p.cpu().numpy() for p in peers], oracle.BF16, want_acc=False)
+            assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), out_want), (M, K, N, P, kr)
+
+
+def test_static_scratch_entry_point_replays_from_a_hip_graph():
+    # the callers it is for include code under HIP graph capture: the call records nothing but its kernel (no clearing of
+    # the scratch: the counters are zero at load and every launch leaves them at zero), so every replay equals the eager result
+    if not torch.cuda.is_available():
+        pytest.fail("GPU test selected but no GPU is visible")
+    so = L.load()
+    g = torch.Generator(device=DEV).manual_seed(11)
+    M, K, N, P, kr = 48, 4096, 1024, 8, 6
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0)
+    x1, x2, s1, s2, bias, peers = _inputs(g, M, K, N, P, kr)
+    d = L.make_desc(0, P, [p.data_ptr() for p in peers], N, 0)
+    d.keptRows = kr
+    need, f, _ = ops.splitk_plan(M, K, N, P, 0, kr)
+    assert f > 1 and need <= L.STATIC_SCRATCH_BYTES
+    out = torch.zeros((kr, N), dtype=torch.bfloat16, device=DEV)
+
+    def call():
+        so.catcoc_launch_quant_matmul_reduce_scatter_static_scratch(
+            torch.cuda.current_stream().cuda_stream, 0, x1.data_ptr(), x2.data_ptr(), s1.data_ptr(), s2.data_ptr(), bias.data_ptr(),
+            None, out.data_ptr(), C.addressof(d), C.byref(t), 0, 0, L.BF16)
+    call()
+    L.check()
+    torch.cuda.synchronize()
+    want = out.clone()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        call()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            out.zero_()
+            call()
+    L.check()
+    for _ in range(3):
+        out.fill_(1.0)
+        call()                                   # eager work between the replays, through the same scratch
+        torch.cuda.synchronize()
+        out.fill_(2.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
 
 
 def test_static_scratch_entry_point_rejects_oversized_launches_and_allocates_nothing():
