@@ -583,6 +583,8 @@ void launch_pipelined(bool quant, int dataType, void *computeStream, void *commS
     g.flags &= ~(uint32_t)GF_RAGGED;   // (ragged problems run the bounds-checked kernel here)
     if (!dma && p.variant == 4) { fail(E_TILING, "m0 = 256 needs full tiles and 16-byte aligned row-major operands"); return; }
     if (!dma && g.transA) p.variant = 0;
+    const bool commWritesOutput = quant && deterministic != 0 && P > 1 && (uintptr_t)scale_x2 % 16 == 0 && (uintptr_t)d_out % 8 == 0;
+    if (dma && commWritesOutput) g.flags |= GF_KEPT_INT32_ONLY;   // (the comm rounds write every kept row's output)
 
     CommArgs c;
     memset(&c, 0, sizeof(c));
@@ -599,6 +601,15 @@ void launch_pipelined(bool quant, int dataType, void *computeStream, void *commS
     c.swizzleDir = 0;
     c.dtype = quant ? (uint32_t)CT_INT32 : outDt;
     const uint32_t cores = splitRow * splitCol;
+    // deterministic W8A8 rounds finish their blocks themselves (int32 sums and the dequantised rows in one pass over them)
+    const bool fuseDequant = commWritesOutput;
+    if (fuseDequant) {
+        c.dOut = d_out;
+        c.ldd = tiling->n;
+        c.scaleN = (const float *)scale_x2;
+        c.scaleM = (const float *)scale_x1 + (size_t)d.rankIdx * sp.mRank;
+        c.outDtype = outDt;
+    }
 
     const uint32_t bpc = sp.blockPerComm, perRank = bpc / P, stages = sp.stages;
     const uint32_t rounds = ceil_div(sp.coreLoops, bpc);
@@ -611,37 +622,43 @@ void launch_pipelined(bool quant, int dataType, void *computeStream, void *commS
             fail(E_WORKSPACE, "this call has %u comm rounds; the plan holds events for %u", rounds, (uint32_t)plan->ready.size());
             return;
         }
-    } else {
+    } else if (rounds > 1 && computeStream != commStream) {   // (a single round, or one stream, needs no event)
         plan = &own;
         if (!plan_make_events(own, rounds)) return;
+    } else {
+        plan = &own;
+        own.ready.assign(rounds, nullptr);
+        own.done.assign(rounds, nullptr);
     }
     std::vector<hipEvent_t> &ready = plan->ready, &done = plan->done;
     hipEvent_t fin = plan->fin;
     auto destroy = [&]() { if (plan == &own) plan_destroy_events(own); };
     hipError_t he = hipSuccess;
-    hipStream_t cs = (hipStream_t)computeStream, ms = (hipStream_t)commStream;
+    // A single round has nothing to overlap: its comm side then runs on computeStream behind the GEMM and no event is needed.
+    const bool oneStream = rounds == 1 || computeStream == commStream;
+    hipStream_t cs = (hipStream_t)computeStream, ms = oneStream ? cs : (hipStream_t)commStream;
     int e = 0;
     for (uint32_t r = 0; r < rounds && e == 0 && he == hipSuccess; ++r) {
         const uint32_t first = r * bpc, actual = umin(bpc, sp.coreLoops - first);
-        if (r >= stages) he = hipStreamWaitEvent(cs, done[r - stages], 0);        // "compute finished" of the stage's last user
+        if (r >= stages && !oneStream) he = hipStreamWaitEvent(cs, done[r - stages], 0);   // "compute finished" of the stage's last user
         g.taskBase = first;
         g.taskCount = actual;
         if (he == hipSuccess)
             e = dma ? (p.dtype == DT_I8 ? launch_gemm_dma_i8(g, computeStream)
                        : p.dtype == DT_F16 ? launch_gemm_dma_f16(g, computeStream) : launch_gemm_dma_bf16(g, computeStream))
                     : launch_gemm(p.dtype, g, p.variant, p.edge, computeStream);
-        if (e == 0 && he == hipSuccess) he = hipEventRecord(ready[r], cs);        // "store finished"
-        if (e == 0 && he == hipSuccess) he = hipStreamWaitEvent(ms, ready[r], 0);
+        if (e == 0 && he == hipSuccess && !oneStream) he = hipEventRecord(ready[r], cs);   // "store finished"
+        if (e == 0 && he == hipSuccess && !oneStream) he = hipStreamWaitEvent(ms, ready[r], 0);
         c.roundFirstIdx = r * perRank;
         c.dataLoops = (actual / P) * (m0 / cb);
-        if (e == 0 && he == hipSuccess && P > 1 && c.dataLoops > 0) e = launch_comm_reduce(c, cores, deterministic != 0, commStream);
-        if (e == 0 && he == hipSuccess) he = hipEventRecord(done[r], ms);
+        if (e == 0 && he == hipSuccess && P > 1 && c.dataLoops > 0) e = launch_comm_reduce(c, cores, deterministic != 0, ms);
+        if (e == 0 && he == hipSuccess && !oneStream) he = hipEventRecord(done[r], ms);
     }
-    if (e == 0 && he == hipSuccess && quant)   // the pass after all rounds: dequantise the reduced int32 block
+    if (e == 0 && he == hipSuccess && quant && !fuseDequant)   // the pass after all rounds: dequantise the reduced int32 block
         e = launch_dequant_rows((const int32_t *)c_accum, tiling->n, (const float *)scale_x2, (const float *)scale_x1 + (size_t)d.rankIdx * sp.mRank,
-                                d_out, tiling->n, sp.mRank, tiling->n, outDt, commStream);
-    if (e == 0 && he == hipSuccess) he = hipEventRecord(fin, ms);
-    if (e == 0 && he == hipSuccess) he = hipStreamWaitEvent(cs, fin, 0);           // the caller's stream sees the finished output
+                                d_out, tiling->n, sp.mRank, tiling->n, outDt, ms);
+    if (e == 0 && he == hipSuccess && !oneStream) he = hipEventRecord(fin, ms);
+    if (e == 0 && he == hipSuccess && !oneStream) he = hipStreamWaitEvent(cs, fin, 0);   // the caller's stream sees the finished output
     destroy();
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
     if (he != hipSuccess) { fail(E_LAUNCH, "stream/event call failed: %s", hipGetErrorString(he)); return; }

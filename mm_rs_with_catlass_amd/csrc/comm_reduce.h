@@ -22,6 +22,15 @@ struct CommArgs {
     uint32_t splitRow, splitCol;   // CommCoreSplit (data split, npu split)
     uint32_t swizzleDir;           // BlockCommSwizzle direction (non-deterministic schedule)
     uint32_t dtype;                // CT_INT32, DT_F16 or DT_BF16
+    // Deterministic int32 rounds can finish their blocks: once a core has added every rank's block the sums are final (a kept
+    // tile belongs to exactly one round), so it writes the dequantised 16-bit rows next to the int32 ones and the pass after
+    // all rounds falls away.  dOut NULL = leave that to the separate pass.
+    void *dOut;                    // [mRank, N] 16-bit output, or NULL
+    int64_t ldd;
+    const float *scaleN;           // per channel, [N]
+    const float *scaleM;           // per token, already at the kept block's first row
+    uint32_t outDtype;             // DT_F16 / DT_BF16
+    uint32_t passes;               // deterministic schedule: pieces of 256 x 4 sixteen-byte accesses a data block is cut into
 };
 
 int launch_comm_reduce(const CommArgs &a, uint32_t cores, bool deterministic, void *stream);

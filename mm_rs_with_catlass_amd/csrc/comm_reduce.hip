@@ -72,12 +72,16 @@ __global__ void __launch_bounds__(256) comm_reduce_kernel(const CommArgs a)
     constexpr uint32_t ES = ELEM == 0 ? 4u : 2u;
 
     if constexpr (DET) {
-        // tasks c, c + cores, ... of the deterministic order are (block c + band * cores, rank sequence): walk blocks
-        for (uint32_t d = blockIdx.x; d < a.dataLoops; d += cores) {
+        // tasks c, c + cores, ... of the deterministic order are (block c + band * cores, rank sequence): walk blocks.  Which
+        // workgroup adds a block does not change any result, so the blocks are dealt out in pieces of 256 x 4 sixteen-byte
+        // accesses (a.passes per block) over as many workgroups as the launch has: more loads in flight per CU.
+        for (uint32_t unit = blockIdx.x; unit < a.dataLoops * a.passes; unit += cores) {
+            const uint32_t d = unit / a.passes;
             const BlockGeom g = block_geom(a, d);
             const uint32_t vecPerRow = g.cols / VEC;                  // (host: n0 and N are multiples of 8)
             const uint32_t total = g.rows * vecPerRow;
-            for (uint32_t e0 = 0; e0 < total; e0 += 256 * 4) {        // up to four 16-byte pieces per thread per pass
+            const uint32_t e0 = (unit - d * a.passes) * (256u * 4u);  // up to four 16-byte pieces per thread per piece
+            if (e0 < total) {
                 v4i acc[4];
                 uint32_t offs[4];
                 bool ok[4];
@@ -124,6 +128,17 @@ __global__ void __launch_bounds__(256) comm_reduce_kernel(const CommArgs a)
                     const uint32_t r = e / vecPerRow, c = e - r * vecPerRow;
                     const size_t lo = ((size_t)(g.row0 + r) * a.localLd + g.col0 + c * VEC) * ES;
                     *(v4i *)((unsigned char *)a.local + lo) = acc[u];
+                    if constexpr (ELEM == 0) {
+                        if (a.dOut != nullptr) {   // the block is final: per-channel scale, then per-token, one rounding
+                            const uint32_t col = g.col0 + c * VEC;
+                            const v4f sn = *(const v4f *)(a.scaleN + col);
+                            const float sm = a.scaleM[g.row0 + r];
+                            uint32_t o[4];
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) o[q] = f32_to_out16(__fmul_rn(__fmul_rn((float)acc[u][q], sn[q]), sm), a.outDtype);
+                            *(v2i *)((unsigned short *)a.dOut + (size_t)(g.row0 + r) * a.ldd + col) = v2i{(int)(o[0] | (o[1] << 16)), (int)(o[2] | (o[3] << 16))};
+                        }
+                    }
                 }
             }
         }
@@ -211,8 +226,16 @@ __global__ void __launch_bounds__(256) reduce_add_kernel(void *dst, const float 
     }
 }
 
-int launch_comm_reduce(const CommArgs &a, uint32_t cores, bool deterministic, void *stream)
+int launch_comm_reduce(const CommArgs &a0, uint32_t cores, bool deterministic, void *stream)
 {
+    CommArgs a = a0;
+    const uint32_t vec = a.dtype == CT_INT32 ? 4u : 8u;
+    a.passes = ceil_div(a.commBlockM * (a.n0 / vec), 256u * 4u);
+    if (a.passes == 0) a.passes = 1;
+    if (deterministic) {   // (the deterministic result does not depend on the number of workgroups)
+        const uint64_t units = (uint64_t)a.dataLoops * a.passes;
+        cores = (uint32_t)(units < 2048u ? (units ? units : 1u) : 2048u);
+    }
     const dim3 grid(cores), block(256);
     hipStream_t s = (hipStream_t)stream;
     if (a.dtype == CT_INT32) {

@@ -21,6 +21,7 @@ enum : uint32_t {
     GF_KEPT_WHOLE = 1u << 5,      // never run kept tiles as two 64-row workgroups
     GF_KEPT_SPLIT = 1u << 6,      // do so whenever the launch allows it (default: by tile count and k length)
     GF_TAIL_WHOLE = 1u << 7,      // never run the tiles that wait for the slots of kept halves as two 64-row workgroups
+    GF_KEPT_INT32_ONLY = 1u << 8, // W8A8, direct-to-LDS kernels: kept tiles store c_accum and nothing else (the caller dequantises later)
     GF_RAGGED = 1u << 4,          // the last tile row of a rank and / or the last tile column are not full: such tiles are computed as
                                   // whole tiles moved up / left so that they end at the edge (they overlap their neighbours, whose
                                   // values they reproduce bit for bit); sums and workspace stores leave the overlap out

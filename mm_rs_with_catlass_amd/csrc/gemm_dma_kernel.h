@@ -927,21 +927,35 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                 }
             }
             if (args.cAccum != nullptr) {
+                // the int32 block, turned around in the wave's 16 KiB of LDS 32 rows at a time like the workspace tiles below:
+                // sixteen-byte stores that cover whole 512-byte row segments instead of 128 four-byte stores per lane
+                static_assert(NW * 16384 <= POOL, "one 16 KiB staging area per wave");
+                unsigned char *stc = smem + w * 16384;
+                __syncthreads();   // every wave has left the main loop's LDS reads behind
+                int32_t *cw = args.cAccum + ((int64_t)(int32_t)out_row0 + wm * 32 * MB) * (int64_t)args.N + ti.col + wn * 128;
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
-                    if (RM && !(keptMb & (1u << mb))) continue;   // (stores only)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const uint32_t lrow = row_base + mb * 32 + (r >> 2) * 8 + (r & 3);
-                        int32_t *o = args.cAccum + (size_t)(uint32_t)(out_row0 + lrow) * args.N + gcol0;
+                        const uint32_t wrow = (r >> 2) * 8 + h * 4 + (r & 3);
 #pragma unroll
                         for (int nb = 0; nb < 4; ++nb) {
                             const int iv = acc[mb][nb][r];
-                            o[32 * nb] = iv;
+                            *(int *)(stc + wrow * 512 + (((nb * 32 + c32) * 4) ^ (h << 7))) = iv;
                         }
+                    }
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const uint32_t wrow = j * 2 + (lane >> 5), chunk = lane & 31;
+                        const v4i v = *(const v4i *)(stc + wrow * 512 + ((chunk * 16) ^ (((wrow >> 2) & 1) << 7)));
+                        if (RM && !(keptMb & (1u << mb))) continue;   // (stores only)
+                        *(v4i *)(cw + (int64_t)(mb * 32 + wrow) * args.N + chunk * 4) = v;
                     }
                 }
             }
+            // a round of the pipelined operator whose comm side also writes the dequantised rows: the int32 block is all
+            // this tile owes
+            if (args.flags & GF_KEPT_INT32_ONLY) return;
             // dequantise in place: per-channel scale first, then per-token, each product rounded on its own
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
