@@ -317,7 +317,7 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
     if (t->m == 0 || t->n == 0 || t->k == 0) return fail(E_SHAPE, "empty problem m=%u n=%u k=%u", t->m, t->n, t->k);
     const uint32_t P = d->rankSize;
     if (P == 0 || P > CATCOC_MAX_RANKS) return fail(E_RANK, "rankSize %u out of range 1..%d", P, CATCOC_MAX_RANKS);
-    if (transA || transB) return fail(E_SHAPE, "the explicit-kept-rows (split-K) path takes row-major A [m,k] and B [k,n] only");
+    if (transA) return fail(E_SHAPE, "the explicit-kept-rows (split-K) path takes A as [m,k] (B as [k,n] or, with transB, as [n,k])");
     if (t->k % 64 != 0 || t->n % 128 != 0)
         return fail(E_SHAPE, "the explicit-kept-rows (split-K) path needs k %% 64 == 0 and n %% 128 == 0 (k=%u, n=%u)", t->k, t->n);
     const bool canLarge = t->m % 128 == 0 && t->n % 256 == 0 && d->keptRowBegin % 32 == 0 && d->keptRows % 32 == 0;
@@ -331,7 +331,6 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
                               "(m0=%u, n0=%u)", t->m0, t->n0);
     if (d->keptRows == 0 || (uint64_t)d->keptRowBegin + d->keptRows > t->m)
         return fail(E_DESC, "kept rows [%u,+%u) outside [0,%u)", d->keptRowBegin, d->keptRows, t->m);
-    if (d->flags & CATCOC_FLAG_REDUCE_INT32) return fail(E_DESC, "the split-K path reduces fp32 peers after the dequant only");
     if ((d->flags & CATCOC_OUTBOUND_MASK) == CATCOC_OUTBOUND_STORE)
         return fail(E_DESC, "the split-K path folds non-kept rows into checksums; CATCOC_OUTBOUND_STORE is not supported there");
     const uint32_t off = d->swizzleOffset ? d->swizzleOffset : 7u;
@@ -341,7 +340,9 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
     GemmArgs &a = sp.args;
     memset(&a, 0, sizeof(a));
     a.M = t->m; a.N = t->n; a.K = t->k;
-    a.lda = t->k; a.ldb = t->n; a.ldd = t->n;
+    a.lda = t->k; a.ldb = transB ? t->k : t->n; a.ldd = t->n;
+    a.transB = transB ? 1 : 0;
+    if (d->flags & CATCOC_FLAG_REDUCE_INT32) a.flags |= GF_REDUCE_INT32;   // int32 peers join the accumulators before the dequant
     a.outDtype = DT_BF16;
     a.sched.off = off; a.sched.dir = dir;
     a.keptBegin = d->keptRowBegin;

@@ -95,7 +95,7 @@ template <uint32_t DT, int WM, bool TB, bool RM, bool RG, bool TA, int MB, int N
 __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *smem, uint32_t pos, uint32_t slice, uint32_t kSlices,
                                          uint32_t subRow)
 {
-    static_assert(!RM || (DT == DT_I8 && WM == 2 && !TB), "row-mask mode exists for the W8A8 128-row kernel");
+    static_assert(!RM || (DT == DT_I8 && WM == 2), "row-mask mode exists for the W8A8 128-row kernel");
     static_assert(!RG || (WM == 2 && !RM), "ragged mode exists for the 128-row kernel");
     static_assert(!TA || (WM == 2 && !RM), "transposed A exists for the 128-row kernel");
     static_assert(WM == 2 || WM == 4, "supported geometries");
@@ -897,8 +897,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
 
     // W8A8 with GF_REDUCE_INT32 (the reference's data flow, quant_matmul_reduce_scatter.hpp:191-201,285-351): the peers'
     // partials are int32 and join the accumulators before the dequantisation; tiles of other ranks leave as raw int32
-    // (explicit kept rows, RM, take fp32 partials only)
-    const bool redI32 = DT == DT_I8 && !RM && (args.flags & GF_REDUCE_INT32) != 0;
+    const bool redI32 = DT == DT_I8 && (args.flags & GF_REDUCE_INT32) != 0;
     const uint32_t nPeersI32 = redI32 ? args.nPeers : 0u, nPeersF32 = redI32 ? 0u : args.nPeers;
     if (kept) {
         // (RM: a tile that starts above keptBegin makes this wrap; it is only added to rows of kept blocks, where the sum
@@ -912,6 +911,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
                     const int32_t *srcb = src + (size_t)(mb * 32) * args.peerLd;
+                    if constexpr (RM) srcb = (keptMb & (1u << mb)) ? srcb : peer + (size_t)(h * 4) * args.peerLd + gcol0;   // (as add_partial)
                     int pv[16][4];
 #pragma unroll
                     for (int r = 0; r < 16; ++r)

@@ -18,7 +18,13 @@ int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
     }
     if (args.flags & GF_ROW_MASK) {   // explicit kept rows in whole 32-row blocks
         const uint32_t wgs = launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u);
-        if (deep_ring(args, wgs, 1u) && deep_ring_pairs(args, 1u))
+        if (args.transB) {   // B as [n,k]: the three-stage and the six-stage ring
+            if (deep_ring(args, wgs, 1u))
+                hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, true, false, false, 6, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);
+            else
+                hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);
+        }
+        else if (deep_ring(args, wgs, 1u) && deep_ring_pairs(args, 1u))
             hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true, false, false, 6, true, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);
         else if (deep_ring(args, wgs, 1u))
             hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true, false, false, 6, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);

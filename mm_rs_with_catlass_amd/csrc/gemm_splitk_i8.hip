@@ -9,11 +9,20 @@ int launch_gemm_splitk_i8(const GemmArgs &args, int rowBlocks, uint32_t tasks, v
     // k slices are whole 256-byte k tiles except the last one, which takes what is left of K: with K a multiple of 128
     // every slice is a whole number of pairs of 64-byte steps, and A can be fetched as whole 128-byte lines
     const bool pairs = args.K % 128u == 0;
-    if (rowBlocks == 1) hipLaunchKernelGGL((gemm_splitk_kernel<1>), grid, block, 0, (hipStream_t)stream, args);
-    else if (rowBlocks == 2 && pairs) hipLaunchKernelGGL((gemm_splitk_kernel<2, true>), grid, block, 0, (hipStream_t)stream, args);
-    else if (rowBlocks == 2) hipLaunchKernelGGL((gemm_splitk_kernel<2>), grid, block, 0, (hipStream_t)stream, args);
-    else if (pairs) hipLaunchKernelGGL((gemm_splitk_kernel<4, true>), grid, block, 0, (hipStream_t)stream, args);
-    else hipLaunchKernelGGL((gemm_splitk_kernel<4>), grid, block, 0, (hipStream_t)stream, args);
+    hipStream_t s = (hipStream_t)stream;
+    if (args.transB) {   // B as [n][k]
+        if (rowBlocks == 1) hipLaunchKernelGGL((gemm_splitk_kernel<1, false, true>), grid, block, 0, s, args);
+        else if (rowBlocks == 2 && pairs) hipLaunchKernelGGL((gemm_splitk_kernel<2, true, true>), grid, block, 0, s, args);
+        else if (rowBlocks == 2) hipLaunchKernelGGL((gemm_splitk_kernel<2, false, true>), grid, block, 0, s, args);
+        else if (pairs) hipLaunchKernelGGL((gemm_splitk_kernel<4, true, true>), grid, block, 0, s, args);
+        else hipLaunchKernelGGL((gemm_splitk_kernel<4, false, true>), grid, block, 0, s, args);
+        return (int)hipGetLastError();
+    }
+    if (rowBlocks == 1) hipLaunchKernelGGL((gemm_splitk_kernel<1>), grid, block, 0, s, args);
+    else if (rowBlocks == 2 && pairs) hipLaunchKernelGGL((gemm_splitk_kernel<2, true>), grid, block, 0, s, args);
+    else if (rowBlocks == 2) hipLaunchKernelGGL((gemm_splitk_kernel<2>), grid, block, 0, s, args);
+    else if (pairs) hipLaunchKernelGGL((gemm_splitk_kernel<4, true>), grid, block, 0, s, args);
+    else hipLaunchKernelGGL((gemm_splitk_kernel<4>), grid, block, 0, s, args);
     return (int)hipGetLastError();
 }
 }  // namespace catcoc

@@ -30,7 +30,10 @@ namespace catcoc {
 // on the way in and masked on the way out.
 // AP: A is fetched per group of two k steps, 128 bytes per row (whole cache lines: half as many requests to L2 as two
 // 64-byte halves), into one "pair" area per group; for 64- and 128-row tiles whose k slices are whole pairs of steps.
-template <int MBW, bool AP = false>
+// TB: B is given as [n][k] (k contiguous, the layout of a stored weight matrix): a step's B stage is then 128 rows of 64
+// bytes of k, copied and read exactly like A's (plain 16-byte fragment reads, no transposing reads).  A line of B is
+// asked for in two halves one step apart; the second finds it in L2, so these copies carry no streaming hint.
+template <int MBW, bool AP = false, bool TB = false>
 __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args)
 {
     static_assert(!AP || MBW >= 2, "pairs of steps are the groups of the 64- and 128-row tiles");
@@ -64,7 +67,23 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
 
     const int64_t lda = args.lda, ldb = args.ldb;
     const unsigned char *Ag = (const unsigned char *)args.a[0] + (size_t)row0 * lda + kBeg;
-    const unsigned char *Bg = (const unsigned char *)args.b + (size_t)kBeg * ldb + colT;
+    const unsigned char *Bg = TB ? (const unsigned char *)args.b + (size_t)colT * ldb + kBeg
+                                 : (const unsigned char *)args.b + (size_t)kBeg * ldb + colT;
+    // B copy j of a step: [k][n] covers k rows 8j..8j+7 (lane -> row 8j + lane/8, slot lane&7 holds chunk slot ^ (((row>>1)&3)<<1));
+    // [n][k] covers tile columns 16j..16j+15, one 64-byte row of k each, laid out like A
+    auto copy_b = [&](const unsigned char *Bgk, unsigned char *sb) {
+#pragma unroll
+        for (int jj = 0; jj < B_CP; ++jj) {
+            const int j = w + NW * jj;
+            if constexpr (TB) {
+                const uint32_t lrow = 16 * j + (lane >> 2);
+                dma16(Bgk + (size_t)lrow * ldb + (((lane & 3) ^ ((lane >> 4) & 3)) * 16), sb + j * 1024);
+            } else {
+                const int row = 8 * j + (lane >> 3);
+                dma16_stream(Bgk + (size_t)row * ldb + (((lane & 7) ^ (((row >> 1) & 3) << 1)) * 16), sb + j * 1024);
+            }
+        }
+    };
 
     // A: copy j covers tile rows 16j..16j+15; lane -> row 16j + lane/4, LDS chunk slot lane&3 holds k chunk slot^swz
     // Every workgroup of a k slice reads the same 64-byte column of A at the same step, and the rows of A are a
@@ -76,7 +95,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         unsigned char *sa = smem + st * STAGE, *sb = sa + A_STAGE;
         const uint32_t kt = step + rot < nsteps ? step + rot : step + rot - nsteps;
         const unsigned char *Agk = Ag + (size_t)kt * 64;
-        const unsigned char *Bgk = Bg + (size_t)kt * 64 * ldb;
+        const unsigned char *Bgk = TB ? Bg + (size_t)kt * 64 : Bg + (size_t)kt * 64 * ldb;
 #pragma unroll
         for (int jj = 0; jj < A_CP; ++jj) {
             const int j = (MBW == 1) ? (w & 1) : w + NW * jj;
@@ -84,13 +103,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
             const uint32_t srow = umin(lrow, rowsValid - 1u);
             dma16(Agk + (size_t)srow * lda + (((lane & 3) ^ ((lane >> 4) & 3)) * 16), sa + j * 1024);
         }
-        // B: copy j covers k rows 8j..8j+7; lane -> row 8j + lane/8, slot lane&7 holds chunk slot ^ (((row>>1)&3)<<1)
-#pragma unroll
-        for (int jj = 0; jj < B_CP; ++jj) {
-            const int j = w + NW * jj;
-            const int row = 8 * j + (lane >> 3);
-            dma16_stream(Bgk + (size_t)row * ldb + (((lane & 7) ^ (((row >> 1) & 3) << 1)) * 16), sb + j * 1024);
-        }
+        copy_b(Bgk, sb);
     };
     // AP: steps `step` and `step + 1` (st even).  The group's area holds the pair of A first (rows of 128 bytes: copy j covers
     // rows 8j..8j+7, lane -> row 8j + lane/8, chunk slot lane&7 holds k chunk slot ^ ((row>>1)&7)), then B of the two steps.
@@ -107,14 +120,8 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const unsigned char *Bgk = Bg + (size_t)(kt + t) * 64 * ldb;
-            unsigned char *sb = sp + 2 * A_STAGE + t * B_STAGE;
-#pragma unroll
-            for (int jj = 0; jj < B_CP; ++jj) {
-                const int j = w + NW * jj;
-                const int row = 8 * j + (lane >> 3);
-                dma16_stream(Bgk + (size_t)row * ldb + (((lane & 7) ^ (((row >> 1) & 3) << 1)) * 16), sb + j * 1024);
-            }
+            const unsigned char *Bgk = TB ? Bg + (size_t)(kt + t) * 64 : Bg + (size_t)(kt + t) * 64 * ldb;
+            copy_b(Bgk, sp + 2 * A_STAGE + t * B_STAGE);
         }
     };
     auto issue_more = [&](uint32_t &issuedSteps) {   // the next step, or the next pair of steps
@@ -212,6 +219,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     // transpose read of this wave's 32 columns (two 16-column chunks, one per half of a 32-lane group)
     const int ti16 = lane & 15, tch = (lane >> 4) & 1, trow = ti16 >> 1, thalf = ti16 & 1;
     const uint32_t b_lds = (16 * h + trow) * 128 + (((2 * w + tch) ^ (((trow >> 1) & 3) << 1)) * 16) + thalf * 8;
+    const uint32_t bt_lds = (w * 32 + c32) * 64;   // [n][k] stage: the row of this lane's column (chunk swizzle a_sw, as for A)
 
     // The loop is paced by latencies, not by bandwidth (one wave per SIMD: barrier, LDS round trip and the MFMA
     // chain of a step add up), so G steps share one barrier and one LDS round trip.  `issued` counts the steps
@@ -249,10 +257,14 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
             const unsigned char *sb = AP ? sa + 2 * A_STAGE + j * B_STAGE : sa + A_STAGE;
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
-                const unsigned char *p = sb + b_lds + kk * 32 * 128;
-                const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
-                const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 128));
-                bf[j][kk] = v4i{t0.x, t0.y, t1.x, t1.y};
+                if constexpr (TB) {
+                    bf[j][kk] = *(const v4i *)(sb + bt_lds + (((2 * kk + h) ^ a_sw) * 16));
+                } else {
+                    const unsigned char *p = sb + b_lds + kk * 32 * 128;
+                    const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
+                    const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 128));
+                    bf[j][kk] = v4i{t0.x, t0.y, t1.x, t1.y};
+                }
 #pragma unroll
                 for (int mb = 0; mb < MBW; ++mb) {
                     if constexpr (AP) af[j][kk][mb] = *(const v4i *)(sa + ap_lds + mb * 32 * 128 + (((4 * j + 2 * kk + h) ^ ap_sw) * 16));
@@ -385,6 +397,9 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     // block it was several times the size of the instruction cache): the block's registers are selected, dequantised,
     // the peers added in slot order eight at a time (the first block's first eight are in registers already, the
     // others are fetched into the same registers in one round trip) and the 16-bit rows stored.
+    // GF_REDUCE_INT32 (the reference's order, quant_matmul_reduce_scatter.hpp:285-351): the peers hold int32 partials that join
+    // the accumulators before the dequantisation, and c_accum receives the reduced block
+    const bool redI32 = (args.flags & GF_REDUCE_INT32) != 0;
     long long csum = csumOthers;
 #pragma unroll
     for (int mb = 0; mb < MBW; ++mb) {
@@ -402,7 +417,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
             for (int r = 0; r < 16; ++r)
                 if (slot_row(r) + vrel < rowsValid) ((int32_t *)args.accDump)[(size_t)(row0 + vrel + slot_row(r)) * N + gcol] = acc[mb][r];
         }
-        if (k.n != 0 && args.cAccum) {
+        if (k.n != 0 && args.cAccum && !redI32) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 if (lane_kept(k, r)) args.cAccum[(size_t)(row0 + vrel + slot_row(r) - args.keptBegin) * N + gcol] = acc[mb][r];
@@ -425,9 +440,25 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
                 for (int r = 0; r < 16; ++r) iv[r] = acc[mb][r];
             }
         float v[16];
+        if (redI32) {
+            for (uint32_t p0 = 0; p0 < args.nPeers; p0 += 8) {
+                if (t != mbK || p0 != 0) fetch_peers(k, p0, pv0);
+#pragma unroll
+                for (int q = 0; q < 8; ++q)
+                    if (p0 + q < args.nPeers) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) iv[r] += f2i(pv0[q][r]);   // (the loads carry bit patterns)
+                    }
+            }
+            if (args.cAccum) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    if (lane_kept(k, r)) args.cAccum[(size_t)(row0 + t * 32 + 4u * h + slot_row(r) - args.keptBegin) * N + gcol] = iv[r];
+            }
+        }
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = __fmul_rn(__fmul_rn((float)iv[r], sN), __shfl(sMt, slot_row(r) + 4 * h, 64));
-        for (uint32_t p0 = 0; p0 < args.nPeers; p0 += 8) {
+        for (uint32_t p0 = 0; p0 < (redI32 ? 0u : args.nPeers); p0 += 8) {
             if (t != mbK || p0 != 0) fetch_peers(k, p0, pv0);
 #pragma unroll
             for (int q = 0; q < 8; ++q)

@@ -200,15 +200,17 @@ def splitk_plan(m, k, n, rank_size, kept_row_begin, kept_rows, split_k=0, block_
 
 def prepare_quant_matmul_splitk(x1, x2, scale_x1, scale_x2, bias=None, peers=(), rank_size=1, kept_row_begin=0,
                                 kept_rows=None, out_dtype=torch.bfloat16, split_k=0, workspace=None, checksum=None,
-                                acc_dump=None, c_accum=None, peer_row_offset=0, block_num=0, swizzle=None, out=None, n0=0):
-    """Skinny-M (decode) form of the W8A8 operator: x1 [m,k] with any m, the rank keeps rows
-    [kept_row_begin, +kept_rows); peers are rank_size-1 fp32 partials [kept_rows, n].  Returns (launch, out)."""
+                                acc_dump=None, c_accum=None, peer_row_offset=0, block_num=0, swizzle=None, out=None, n0=0,
+                                trans_b=False, reduce_int32=False):
+    """Skinny-M (decode) form of the W8A8 operator: x1 [m,k] with any m, x2 [k,n] (or [n,k] with trans_b, the layout of a
+    stored weight matrix), the rank keeps rows [kept_row_begin, +kept_rows); peers are rank_size-1 partials [kept_rows, n],
+    fp32 added after the dequantisation or, with reduce_int32, int32 added before it.  Returns (launch, out)."""
     _check_rank(0, rank_size)
     _want(x1, "x1", torch.int8, 2)
     _want(x2, "x2", torch.int8, 2)
     m, k = x1.shape
-    n = x2.shape[1]
-    if x2.shape[0] != k:
+    n = x2.shape[0] if trans_b else x2.shape[1]
+    if (x2.shape[1] if trans_b else x2.shape[0]) != k:
         _fail("x2 has shape %s: its k extent does not match x1's k = %d", tuple(x2.shape), k)
     kr = kept_rows if kept_rows is not None else m
     if kept_row_begin < 0 or kr < 1 or kept_row_begin + kr > m:
@@ -218,14 +220,15 @@ def prepare_quant_matmul_splitk(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
     _want(scale_x1, "scale_x1", torch.float32, 1, m)
     _want(scale_x2, "scale_x2", torch.float32, 1, n)
     _want(bias, "bias", torch.int32, 1, n)
-    _check_peers(list(peers), rank_size - 1, torch.float32, peer_row_offset + kr, n)
+    _check_peers(list(peers), rank_size - 1, torch.int32 if reduce_int32 else torch.float32, peer_row_offset + kr, n)
     _want(c_accum, "c_accum", torch.int32, None, kr * n)
     _want(acc_dump, "acc_dump", torch.int32, None, m * n)
     _want(checksum, "checksum", torch.int64, None, -(-m // 128) * -(-n // 128))
     _want(out, "out", (torch.float16, torch.bfloat16), 2, None, (kr, n))
     _check_dev(x1, x2, scale_x1, scale_x2, bias, checksum, acc_dump, c_accum, workspace, out, *peers)
     t = default_tiling(m, k, n, rank_size, m0=128 if n0 else 0, n0=n0, k0=0)
-    d = _desc(0, rank_size, list(peers), peer_row_offset, 0, block_num, 0, swizzle, None, checksum, acc_dump)
+    d = _desc(0, rank_size, list(peers), peer_row_offset, _l.FLAG_REDUCE_INT32 if reduce_int32 else 0, block_num, 0, swizzle, None,
+              checksum, acc_dump)
     d.keptRowBegin = kept_row_begin
     d.keptRows = kept_rows if kept_rows is not None else m
     d.splitK = split_k
@@ -237,7 +240,7 @@ def prepare_quant_matmul_splitk(x1, x2, scale_x1, scale_x2, bias=None, peers=(),
     keep = (x1, x2, scale_x1, scale_x2, bias, tuple(peers), checksum, acc_dump, c_accum, out, d, t, workspace)
     fn = _l.load().catcoc_launch_quant_matmul_reduce_scatter
     argv = (0, x1.data_ptr(), x2.data_ptr(), scale_x1.data_ptr(), scale_x2.data_ptr(), _ptr(bias), _ptr(c_accum),
-            out.data_ptr(), C.addressof(d), C.byref(t), 0, 0, _TORCH_TO_DT[out.dtype])
+            out.data_ptr(), C.addressof(d), C.byref(t), 0, int(trans_b), _TORCH_TO_DT[out.dtype])
 
     def launch(_keep=keep):
         fn(_stream(), *argv)

@@ -457,6 +457,45 @@ def test_quant_skinny_m_splitk(case):
         assert cs[t] == blk[~keep[mi * 128:(mi + 1) * 128]].sum(), t
 
 
+@pytest.mark.parametrize("case", [(1, 8192, 8192, 8, 0, 1), (16, 8192, 8192, 8, 0, 2), (128, 8192, 8192, 8, 16, 16), (64, 1024, 4160, 4, 40, 24),
+                                  (512, 8192, 8192, 8, 64, 64), (100, 384, 1088, 2, 3, 90)])
+@pytest.mark.parametrize("mode", ["weights_n_by_k", "int32_reduce", "both"])
+def test_quant_skinny_m_weight_layout_and_reference_reduce_order(case, mode):
+    """The decode path in the layouts and modes the reference uses: B stored as [n,k] (transB, the layout of its sweep shapes,
+    examples/dynamic_tiling/scripts/test_shapes.csv, and of a weight matrix) and int32 peers that join the accumulators before
+    the dequantisation (quant_matmul_reduce_scatter.hpp:285-351), at K = N = 8192 for M = 1, 16, 128 and 512 (the large-tile
+    route) and on odd shapes.  Accumulators, reduced int32 block and output bit for bit against the oracle."""
+    _need_gpu()
+    M, N, K, P, kb, kr = case
+    tb, ri = mode != "int32_reduce", mode != "weights_n_by_k"
+    rng = np.random.default_rng(260 + M)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.integers(-1000, 1000, N, dtype=np.int32)
+    if ri:
+        peers = [rng.integers(-2 ** 24, 2 ** 24, (kr, N), dtype=np.int32) for _ in range(P - 1)]
+    else:
+        peers = [rng.standard_normal((kr, N)).astype(np.float32) for _ in range(P - 1)]
+    acc_k, out_want = oracle.quant_matmul_reduce_scatter(x1[kb:kb + kr], x2, s1[kb:kb + kr], s2, b, 0, kr, peers, oracle.BF16, reduce_int32=ri)
+    need, fac, tiles = ops.splitk_plan(M, K, N, P, kb, kr)
+    ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=DEV)
+    c_accum = torch.full((kr, N), -7, dtype=torch.int32, device=DEV)
+    x2d = dev(np.ascontiguousarray(x2.T)) if tb else dev(x2)
+    launch, out = ops.prepare_quant_matmul_splitk(dev(x1), x2d, dev(s1), dev(s2), dev(b), [dev(p) for p in peers], P, kb, kr,
+                                                  workspace=ws, c_accum=c_accum, trans_b=tb, reduce_int32=ri)
+    for it in range(2):
+        out.zero_()
+        launch()
+        L.check()
+        torch.cuda.synchronize()
+        kept = acc_k + (sum(peers) if ri else 0)
+        assert np.array_equal(c_accum.cpu().numpy(), kept), "kept int32 block differs from the oracle"
+        assert np.array_equal(host16(out), out_want), "kept rows differ from the oracle"
+    assert not ws[:65536].any()
+
+
 @pytest.mark.parametrize("case", [(64, 256, 4096, 8, 8, 8, 0), (128, 640, 2048, 8, 112, 16, 0), (200, 256, 1088, 4, 100, 50, 3),
                                   (100, 384, 1024, 8, 37, 13, 4), (256, 256, 2048, 2, 130, 60, 2), (33, 128, 512, 2, 0, 33, 2),
                                   (128, 256, 1024, 1, 0, 128, 4), (190, 128, 768, 8, 0, 5, 3)])
