@@ -81,6 +81,7 @@ def decode_sweep(args, torch, L, ops, dev):
     P, copies = 8, 6
     g = torch.Generator(device=dev).manual_seed(20250101)
     Bs = [torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev, generator=g) for _ in range(copies)]
+    Bts = [b.t().contiguous() for b in Bs]
     s2 = torch.empty(N, device=dev).uniform_(0.001, 0.01, generator=g)
     sweep = []
     for M in (1, 16, 64, 128, 512):
@@ -91,30 +92,37 @@ def decode_sweep(args, torch, L, ops, dev):
         need, f, tiles = ops.splitk_plan(M, K, N, P, 0, kr)
         ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=dev)
         out = torch.empty((kr, N), dtype=torch.bfloat16, device=dev)
-        steps = [ops.prepare_quant_matmul_splitk(x1, b, s1, s2, None, peers, P, 0, kr, workspace=ws, out=out)[0] for b in Bs]
-        steps[0]()
-        L.check()
-        for i in range(args.warmup):
-            steps[i % copies]()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record()
-        for i in range(args.steps):
-            steps[i % copies]()
-        e1.record()
-        torch.cuda.synchronize()
-        wall = (time.perf_counter() - t0) / args.steps
-        kern = e0.elapsed_time(e1) / args.steps / 1e3
+        def timed(steps):
+            steps[0]()
+            L.check()
+            for i in range(args.warmup):
+                steps[i % copies]()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            e0.record()
+            for i in range(args.steps):
+                steps[i % copies]()
+            e1.record()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / args.steps, e0.elapsed_time(e1) / args.steps / 1e3
+        # the same weights stored as [n,k] (transB, the layout of the reference's sweep shapes), timed first; the row-major
+        # run comes last, so that `out` holds what the parity check below compares
+        wall_t, kern_t = timed([ops.prepare_quant_matmul_splitk(x1, bt, s1, s2, None, peers, P, 0, kr, workspace=ws, out=out, trans_b=True)[0]
+                                for bt in Bts])
+        out_t = out.clone()
+        wall, kern = timed([ops.prepare_quant_matmul_splitk(x1, b, s1, s2, None, peers, P, 0, kr, workspace=ws, out=out)[0] for b in Bs])
         # parity of the last launch (B copy (steps-1) % copies) against the oracle
         bl = Bs[(args.steps - 1) % copies]
         _, want = oracle.quant_matmul_reduce_scatter(x1[:kr].cpu().numpy(), bl.cpu().numpy(), s1[:kr].cpu().numpy(), s2.cpu().numpy(),
                                                      None, 0, kr, [p.cpu().numpy() for p in peers], oracle.BF16, want_acc=False)
-        ok = bool(np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), want))
+        ok = bool(np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), want)) and bool(torch.equal(out_t.view(torch.int16), out.view(torch.int16)))
         alg = K * N + M * K + 4 * (M + N) + (P - 1) * kr * N * 4 + kr * N * 2
         sweep.append({"M": M, "kept_rows": kr, "split_k": f, "tiles": tiles, "kernel_us": round(kern * 1e6, 2),
                       "wall_us": round(wall * 1e6, 2), "algorithmic_bytes": alg, "GBps": round(alg / kern / 1e9, 1),
                       "hbm_frac": round(alg / kern / 1e9 / PEAK_HBM_GBS, 4), "TOPS": round(2.0 * M * N * K / kern / 1e12, 2),
+                      "weights_n_by_k": {"kernel_us": round(kern_t * 1e6, 2), "GBps": round(alg / kern_t / 1e9, 1),
+                                         "TOPS": round(2.0 * M * N * K / kern_t / 1e12, 2)},
                       "parity_ok": ok})
     hbm = [r for r in sweep if r["M"] <= 128]
     worst = min(hbm, key=lambda r: r["GBps"])

@@ -218,20 +218,23 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
 
     // Few tiles: the 128-row direct-to-LDS kernel can cut every tile's k range into slices, one workgroup each, that
     // meet through a workspace (partial tiles [tiles][slices][128*256] as 32-bit words, then one counter per tile).
-    // Chosen so that the slices fill the 256 CUs once, each with at least eight k steps; float partials are limited to
-    // two slices (their sum does not depend on which arrives last).  desc.splitK overrides the choice.
+    // Chosen so that the slices fill the 256 CUs once, each with at least eight k steps; float launches take
+    // two slices by themselves (see fauto below).  desc.splitK overrides the choice.
     plan.kSlices = 1;
     plan.kSliceBytes = 0;
     if (plan.dma && !plan.edge && m0 == 128 && d->keptRows == 0) {
         const uint32_t T = a.sched.coreLoops, nkAll = (uint32_t)((uint64_t)t->k * es / 64u);
-        const uint32_t fmax = dt == DT_I8 ? 8u : 2u;
+        const uint32_t fmax = 8u;
+        // the library's own choice stays at two slices for float operands (more are reproducible too -- three or more float
+        // partials are added in slice order -- but did not measure faster: the last slice then fetches every partial)
+        const uint32_t fauto = dt == DT_I8 ? 8u : 2u;
         uint32_t f = 1;
         if (d->splitK != 0) {
             if (d->splitK > fmax || d->splitK > nkAll)
-                return fail(E_TILING, "splitK %u: at most %u k slices for this element type and k", d->splitK, umin(fmax, nkAll));
+                return fail(E_TILING, "splitK %u: at most %u k slices for this k", d->splitK, umin(fmax, nkAll));
             f = d->splitK;
         } else {
-            while (f * 2u <= fmax && T * f * 2u <= 256u && nkAll / (f * 2u) >= 8u) f *= 2u;
+            while (f * 2u <= fauto && T * f * 2u <= 256u && nkAll / (f * 2u) >= 8u) f *= 2u;
         }
         if (f > 1) {
             plan.kSlices = f;

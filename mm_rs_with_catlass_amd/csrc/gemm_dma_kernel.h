@@ -688,8 +688,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     // Every slice writes its partial tile through to memory (device-scope stores, 16 bytes per lane, the tile in
     // register order: index (((mb*4 + nb)*4 + g)*256 + thread)*4 + j holds register r = 4g + j), a per-tile counter
     // elects the last slice to arrive, and that workgroup adds the others' partials and goes on to the epilogue.
-    // Integer partials add exactly in any order; float partials are limited to two slices by the host, whose sum
-    // does not depend on which of them arrives last.
+    // (the order of the additions: below, where the partials meet)
     // RM: only the 32-row blocks with kept rows travel (unless the caller wants a dump of every accumulator): of the others
     // a checksum needs the sum alone, and sums of sums are exact, so every lane adds up what it holds of such a block and
     // the eight bytes travel in the place of the block's first 16.  At M = 512 with 64 kept rows three tiles in four then
@@ -742,8 +741,25 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             __syncthreads();
             if (*flag != kSlices - 1u) return;
             if (tid == 0) __hip_atomic_store(args.skCount + task, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            for (uint32_t o = 0; o + 1 < kSlices; ++o) {
-                const uint32_t sl = o < slice ? o : o + 1;
+            // Integer partials add exactly in any order, and so do two float partials: the last slice to arrive keeps its own in
+            // registers and adds the others.  Three or more float partials are added in SLICE order whichever slice arrives
+            // last (the result then does not depend on timing): the accumulators restart at zero and every slice's partial,
+            // the workgroup's own included, comes back from the workspace, slice 0 first.
+            const bool ordered = DT != DT_I8 && kSlices > 2u;
+            if constexpr (DT != DT_I8) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const float keep = acc[mb][nb][r];
+                            acc[mb][nb][r] = ordered ? 0.0f : keep;   // (a select, not a branch around the accumulators)
+                        }
+            }
+            const uint32_t nOthers = ordered ? kSlices : kSlices - 1u;
+            for (uint32_t o = 0; o < nOthers; ++o) {
+                const uint32_t sl = ordered ? o : (o < slice ? o : o + 1);
                 const __amdgpu_buffer_rsrc_t other = __builtin_amdgcn_make_buffer_rsrc(
                     (void *)(args.skPart + ((size_t)task * kSlices + sl) * TILE_WORDS), 0, (int)(TILE_WORDS * 4), 0x00020000);
 #pragma unroll

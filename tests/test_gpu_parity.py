@@ -400,8 +400,8 @@ def test_k_slice_rejections():
     _need_gpu()
     a = torch.zeros((512, 1024), dtype=torch.float16, device=DEV)
     b = torch.zeros((1024, 1024), dtype=torch.float16, device=DEV)
-    with pytest.raises(L.CatcocError, match="at most 2 k slices"):
-        ops.matmul_allreduce(a, b, [], 0, 1, split_k=4, workspace=torch.zeros(1 << 24, dtype=torch.uint8, device=DEV))
+    with pytest.raises(L.CatcocError, match="at most 8 k slices"):
+        ops.matmul_allreduce(a, b, [], 0, 1, split_k=16, workspace=torch.zeros(1 << 24, dtype=torch.uint8, device=DEV))
     with pytest.raises(L.CatcocError, match="needs a workspace"):
         ops.matmul_allreduce(a, b, [], 0, 1, split_k=2)
     with pytest.raises(L.CatcocError, match="workspace too small"):
@@ -899,6 +899,23 @@ def test_float_few_tiles_k_sliced(dtype):
     out = ops.matmul_allreduce(dev16(A, dtype), dev16(B, dtype), [dev(fullp[0])], 0, 2, workspace=ws)
     torch.cuda.synchronize()
     _check_float(host16(out), want, part + fullp[0], dtype, K)
+    # three and more slices (the caller's choice): their fp32 partials are added in slice order whichever slice arrives last,
+    # so repeated launches still agree bit for bit, outputs and dumped partials alike
+    for f in (3, 4, 8):
+        need, got_f = ops.kslice_plan(L.MATMUL_ALLREDUCE, tdt, M, K, N, 0, 2, split_k=f)
+        assert got_f == f
+        ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+        outs, dumps = [], []
+        for _ in range(3):
+            dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+            out = ops.matmul_allreduce(dev16(A, dtype), dev16(B, dtype), [dev(fullp[0])], 0, 2, workspace=ws, split_k=f, acc_dump=dump)
+            torch.cuda.synchronize()
+            outs.append(host16(out))
+            dumps.append(dump.cpu().numpy())
+        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2]), f
+        assert np.array_equal(dumps[0], dumps[1]) and np.array_equal(dumps[0], dumps[2]), f
+        _check_float(outs[0], want, part + fullp[0], dtype, K)
+        assert not ws[:65536].any()
 
 
 @pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
