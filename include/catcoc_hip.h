@@ -303,8 +303,9 @@ CATCOC_API uint64_t catcoc_get_workspace_size(int commType, int dataType, const 
  * by the caller, re-armed by every launch): returns the bytes needed and the slice count (1 and 0 bytes when the
  * launch would not be sliced: other tile shapes, ragged problems, enough tiles already; the operands' layouts do
  * not matter).  The count
- * is 2, 4 or 8 for W8A8 (integer partials add exactly) and at most 2 for fp16/bf16 (a two-term fp32 sum does not
- * depend on which slice arrives last); desc->splitK, when non-zero, is taken as the caller's own count.  A launch
+ * is 2, 4 or 8 for W8A8 (integer partials add exactly) and 2 for fp16/bf16; desc->splitK, when non-zero, is taken as the
+ * caller's own count (up to 8; three or more fp32 partials are added in slice order whichever slice arrives last, so
+ * the result is reproducible for any count).  A launch
  * slices only when `workspace` is given.  Counterpart in the reference: SplitkMatmul's k split
  * (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:68-148), which its communication kernels do not
  * use. */
@@ -313,10 +314,13 @@ CATCOC_API uint64_t catcoc_get_kslice_workspace_size(int commType, int dataType,
 
 /* Split-K path (descriptor with keptRows != 0): bytes of `workspace` the launch needs (0 when the split factor
  * is 1), the split factor it will use and its number of 128x128 tiles (`checksum`, if given, needs one int64 per
- * tile and receives the sum of the accumulators of the tile's rows that are not kept).  The path takes row-major
- * int8 A [m,k] and B [k,n], k % 64 == 0, n % 128 == 0, fp32 peers [keptRows, n].  It stands in for
- * SplitkMatmul (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:68-330) in front of the
- * dequant / reduce epilogue. */
+ * tile and receives the sum of the accumulators of the tile's rows that are not kept).  The path takes int8 A [m,k]
+ * and B [k,n] (or, with transB, [n,k]: a weight matrix stored output-major), peers [keptRows, n] as fp32 added after
+ * the dequantisation or, with CATCOC_FLAG_REDUCE_INT32, int32 added before it.  k in whole 64-byte steps and n in whole
+ * 128-column tiles run the streaming kernels; any other k or n runs whole tiles on a one-thread-per-element kernel
+ * (correct, slow, no k split).  CATCOC_OUTBOUND_STORE does not apply (explicit kept rows have no rank structure to lay
+ * tiles out by).  It stands in for SplitkMatmul (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:68-330)
+ * in front of the dequant / reduce epilogue. */
 CATCOC_API uint64_t catcoc_get_splitk_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,
                                                      uint32_t *splitK, uint32_t *tiles);
 

@@ -299,6 +299,7 @@ struct SplitkPlan {
     GemmArgs args;
     uint32_t f, tiles, rowBlocks;
     uint64_t workspaceBytes;   // partial tiles + counters (0 when f == 1)
+    bool general;              // shape outside the fast routes: gemm_general_kernel on the 128x128 grid
     bool large;                // many rows: the 128x256 direct-to-LDS kernel in row-mask mode runs instead of the split-K kernel
 };
 
@@ -321,9 +322,10 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
     const uint32_t P = d->rankSize;
     if (P == 0 || P > CATCOC_MAX_RANKS) return fail(E_RANK, "rankSize %u out of range 1..%d", P, CATCOC_MAX_RANKS);
     if (transA) return fail(E_SHAPE, "the explicit-kept-rows (split-K) path takes A as [m,k] (B as [k,n] or, with transB, as [n,k])");
-    if (t->k % 64 != 0 || t->n % 128 != 0)
-        return fail(E_SHAPE, "the explicit-kept-rows (split-K) path needs k %% 64 == 0 and n %% 128 == 0 (k=%u, n=%u)", t->k, t->n);
-    const bool canLarge = t->m % 128 == 0 && t->n % 256 == 0 && d->keptRowBegin % 32 == 0 && d->keptRows % 32 == 0;
+    // shapes the two fast routes cannot take (k not in whole 64-byte steps, n not in whole 128-column tiles) run the
+    // one-thread-per-element kernel on the same 128x128 grid: a correctness path, whole tiles, no workspace
+    sp.general = t->k % 64 != 0 || t->n % 128 != 0;
+    const bool canLarge = !sp.general && t->m % 128 == 0 && t->n % 256 == 0 && d->keptRowBegin % 32 == 0 && d->keptRows % 32 == 0;
     const bool wantLarge = t->n0 == 256 && (t->m0 == 0 || t->m0 == 128);
     if (wantLarge && !canLarge)
         return fail(E_TILING, "128x256 tiles with explicit kept rows need m %% 128 == 0, n %% 256 == 0 and kept rows in whole 32-row blocks "
@@ -366,7 +368,18 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
 
     const uint32_t cores = d->blockNum ? d->blockNum : kDefaultBlockNum;
     const uint32_t kTiles = ceil_div(t->k, 256u);
-    sp.tiles = ceil_div(t->m, 128u) * (t->n / 128u);
+    sp.tiles = ceil_div(t->m, 128u) * ceil_div(t->n, 128u);
+    if (sp.general) {
+        if (d->splitK > 1) return fail(E_TILING, "k %% 64 != 0 or n %% 128 != 0: this shape runs whole tiles on the general kernel; splitK %u is not available", d->splitK);
+        const uint32_t stages = d->workspaceStages ? d->workspaceStages : kDefaultStages;
+        a.sched = make_sched(OP_ALLREDUCE, t->m, t->n, 1, 128, 128, cores, 1, stages, off, dir);
+        a.flags |= GF_ROW_MASK;
+        sp.f = 1;
+        a.splitK = 0;
+        sp.rowBlocks = 4;
+        sp.workspaceBytes = 0;
+        return 0;
+    }
     if (sp.large) {
         // one grid of 128x256 tiles over all of A's rows (no rank structure), k slices as for any few-tile launch
         const uint32_t stages = d->workspaceStages ? d->workspaceStages : kDefaultStages;
@@ -407,11 +420,21 @@ void launch_quant_splitk(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_
     if (make_splitk_plan(tiling, d, transA, transB, sp)) return;
     if (!x1 || !x2 || !scale_x1 || !scale_x2 || !d_out) { fail(E_NULL, "x1, x2, scale_x1, scale_x2 and d_out must be non-NULL"); return; }
     if (outDataType != FP16 && outDataType != BF16) { fail(E_DTYPE, "outDataType %u must be FP16 (1) or BF16 (27)", outDataType); return; }
+    GemmArgs &a = sp.args;
+    if (sp.general) {
+        a.a[0] = x1; a.b = x2; a.d = d_out;
+        a.scaleM = (const float *)scale_x1; a.scaleN = (const float *)scale_x2;
+        a.bias = (const int32_t *)bias; a.cAccum = (int32_t *)c_accum;
+        a.outDtype = outDataType;
+        const int eg = launch_gemm(DT_I8, a, 0, true, stream);
+        if (eg) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)eg)); return; }
+        ok();
+        return;
+    }
     if ((uintptr_t)x1 % 16 != 0 || (uintptr_t)x2 % 16 != 0 || sp.args.lda % 16 != 0 || sp.args.ldb % 16 != 0) {
         fail(E_SHAPE, "the split-K path needs 16-byte aligned x1, x2 and row pitches");
         return;
     }
-    GemmArgs &a = sp.args;
     // The large-tile route picked its k slices by itself (no desc.splitK): they need a workspace to meet through, and without
     // one that fits the tiles run whole, as any other few-tile launch of that kernel does.  Only an explicit splitK insists.
     if (sp.large && sp.f > 1 && d->splitK == 0 &&

@@ -505,8 +505,12 @@ __global__ void __launch_bounds__(256) gemm_general_kernel(const GemmArgs args)
     if (!task_tile(sp, task, ti)) return;
     const bool gather = sp.op == OP_ALLGATHER;
     const uint32_t arow0 = gather ? ti.rowInRank : ti.row;
-    const bool kept = ti.row >= args.keptBegin && ti.row < args.keptBegin + args.keptRows;
-    const uint32_t keptLeft = kept ? args.keptBegin + args.keptRows - ti.row : 0;
+    // GF_ROW_MASK (explicit kept rows, which need not line up with tiles): every row decides for itself, and `checksum` takes
+    // the rows that are not kept per tile of the plain grid, index (row / m0) * ceil(N / n0) + col / n0
+    const bool rowMask = (args.flags & GF_ROW_MASK) != 0;
+    const bool kept = rowMask ? (ti.row < args.keptBegin + args.keptRows && ti.row + ti.rowsValid > args.keptBegin)
+                              : (ti.row >= args.keptBegin && ti.row < args.keptBegin + args.keptRows);
+    const uint32_t keptLeft = kept && !rowMask ? args.keptBegin + args.keptRows - ti.row : 0;
     __shared__ double red[256];
     double csum = 0.0;
     long long isum = 0;
@@ -548,7 +552,8 @@ __global__ void __launch_bounds__(256) gemm_general_kernel(const GemmArgs args)
             if constexpr (DT == DT_I8) ((int32_t *)args.accDump)[o] = iacc;
             else ((float *)args.accDump)[o] = facc;
         }
-        if (kept && lrow < keptLeft) {
+        const bool rowKept = rowMask ? (ti.row + lrow - args.keptBegin) < args.keptRows : (kept && lrow < keptLeft);   // (unsigned: rows above keptBegin wrap)
+        if (rowKept) {
             const uint32_t orow = ti.row - args.keptBegin + lrow;
             float v;
             if constexpr (DT == DT_I8) {
@@ -580,7 +585,8 @@ __global__ void __launch_bounds__(256) gemm_general_kernel(const GemmArgs args)
             else csum += (double)facc;
         }
     }
-    if (!kept && !(args.flags & GF_OUTBOUND_STORE) && args.checksum != nullptr) {
+    if ((!kept || rowMask) && !(args.flags & GF_OUTBOUND_STORE) && args.checksum != nullptr) {
+        const size_t slot = rowMask ? (size_t)(ti.row / sp.m0) * sp.loopsN + ti.col / sp.n0 : (size_t)task;
         if constexpr (DT == DT_I8) ((long long *)red)[threadIdx.x] = isum;
         else red[threadIdx.x] = csum;
         __syncthreads();
@@ -588,11 +594,11 @@ __global__ void __launch_bounds__(256) gemm_general_kernel(const GemmArgs args)
             if constexpr (DT == DT_I8) {
                 long long t = 0;
                 for (int i = 0; i < 256; ++i) t += ((long long *)red)[i];
-                ((long long *)args.checksum)[task] = t;
+                ((long long *)args.checksum)[slot] = t;
             } else {
                 double t = 0;
                 for (int i = 0; i < 256; ++i) t += red[i];
-                ((double *)args.checksum)[task] = t;
+                ((double *)args.checksum)[slot] = t;
             }
         }
     }

@@ -258,8 +258,12 @@ def test_workspace_size_queries(so):
     assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024, 4096, 1024, 0, 8) == (32 * 8 * 131072 + 65536, 8)
     assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024, 4096, 1024, 0, 8, split_k=2)[1] == 2
     assert ops.kslice_plan(L.QUANT_MATMUL_REDUCE_SCATTER, torch.int8, 1024 + 8, 4096, 1024, 0, 8) == (0, 1)   # ragged rows
-    with pytest.raises(L.CatcocError, match="at most 2 k slices"):
-        ops.kslice_plan(L.MATMUL_ALLREDUCE, torch.float16, 512, 1024, 1024, 0, 2, split_k=4)
+    # the caller's own count: up to eight for floats too (three or more partials are added in slice order)
+    assert ops.kslice_plan(L.MATMUL_ALLREDUCE, torch.float16, 512, 1024, 1024, 0, 2, split_k=4) == (16 * 4 * 131072 + 65536, 4)
+    with pytest.raises(L.CatcocError, match="at most 8 k slices"):
+        ops.kslice_plan(L.MATMUL_ALLREDUCE, torch.float16, 512, 1024, 1024, 0, 2, split_k=16)
+    # explicit kept rows on a shape outside the streaming kernels (k not in 64-byte steps): whole tiles, no workspace
+    assert ops.splitk_plan(40, 100, 200, 4, 5, 20) == (0, 1, 2)
     need, f, tiles = ops.splitk_plan(16, 8192, 8192, 8, 0, 2)
     assert (f, tiles) == (oracle.splitk_factor(16, 8192, 8192, 256, 128, 128, 256), 64)
     assert need == f * tiles * 128 * 128 * 4 + 65536    # counter block of a fixed size first, then the partial tiles

@@ -496,6 +496,47 @@ def test_quant_skinny_m_weight_layout_and_reference_reduce_order(case, mode):
     assert not ws[:65536].any()
 
 
+@pytest.mark.parametrize("case", [(40, 200, 100, 4, 5, 20, False, False), (130, 264, 192, 2, 100, 30, True, False), (17, 128, 72, 8, 0, 17, False, True),
+                                  (260, 136, 1000, 4, 120, 140, True, True)])
+def test_quant_explicit_kept_rows_on_odd_shapes(case):
+    # k that is not whole 64-byte steps or n that is not whole 128-column tiles: the explicit-kept-rows launch runs the
+    # one-thread-per-element kernel on the same 128x128 grid (kept rows need not line up with tiles); everything it writes
+    # against the oracle: accumulators, kept int32 block, output, checksums of the rows that are not kept
+    _need_gpu()
+    M, N, K, P, kb, kr, tb, ri = case
+    rng = np.random.default_rng(360 + M)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.integers(-1000, 1000, N, dtype=np.int32)
+    peers = [rng.integers(-2 ** 24, 2 ** 24, (kr, N), dtype=np.int32) if ri else rng.standard_normal((kr, N)).astype(np.float32) for _ in range(P - 1)]
+    acc_want, out_want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, b, kb, kr, peers, oracle.BF16, reduce_int32=ri)
+    need, fac, tiles = ops.splitk_plan(M, K, N, P, kb, kr)
+    assert need == 0 and fac == 1 and tiles == -(-M // 128) * -(-N // 128)
+    acc_dump = torch.full((M, N), -7, dtype=torch.int32, device=DEV)
+    c_accum = torch.full((kr, N), -7, dtype=torch.int32, device=DEV)
+    checksum = torch.zeros(tiles, dtype=torch.int64, device=DEV)
+    x2d = dev(np.ascontiguousarray(x2.T)) if tb else dev(x2)
+    out = ops.quant_matmul_splitk(dev(x1), x2d, dev(s1), dev(s2), dev(b), [dev(p) for p in peers], P, kb, kr, checksum=checksum,
+                                  acc_dump=acc_dump, c_accum=c_accum, trans_b=tb, reduce_int32=ri)
+    torch.cuda.synchronize()
+    assert np.array_equal(acc_dump.cpu().numpy(), acc_want)
+    assert np.array_equal(c_accum.cpu().numpy(), acc_want[kb:kb + kr] + (sum(peers) if ri else 0))
+    assert np.array_equal(host16(out), out_want)
+    cs = checksum.cpu().numpy()
+    keep = np.zeros(M, bool)
+    keep[kb:kb + kr] = True
+    nt = -(-N // 128)
+    for t in range(tiles):
+        mi, ni = divmod(t, nt)
+        blk = acc_want[mi * 128:(mi + 1) * 128, ni * 128:(ni + 1) * 128].astype(np.int64)
+        assert cs[t] == blk[~keep[mi * 128:(mi + 1) * 128]].sum(), t
+    with pytest.raises(L.CatcocError, match="runs whole tiles on the general kernel"):
+        ops.quant_matmul_splitk(dev(x1), x2d, dev(s1), dev(s2), dev(b), [dev(p) for p in peers], P, kb, kr, trans_b=tb, reduce_int32=ri,
+                                split_k=2, workspace=torch.zeros(1 << 20, dtype=torch.uint8, device=DEV))
+
+
 @pytest.mark.parametrize("case", [(64, 256, 4096, 8, 8, 8, 0), (128, 640, 2048, 8, 112, 16, 0), (200, 256, 1088, 4, 100, 50, 3),
                                   (100, 384, 1024, 8, 37, 13, 4), (256, 256, 2048, 2, 130, 60, 2), (33, 128, 512, 2, 0, 33, 2),
                                   (128, 256, 1024, 1, 0, 128, 4), (190, 128, 768, 8, 0, 5, 3)])
@@ -537,12 +578,8 @@ def test_quant_skinny_m_splitk_checksums_without_dump(case):
 
 def test_quant_skinny_m_rejections():
     _need_gpu()
-    x1 = torch.zeros((16, 96), dtype=torch.int8, device=DEV)
-    x2 = torch.zeros((96, 256), dtype=torch.int8, device=DEV)
     s1 = torch.ones(16, device=DEV)
     s2 = torch.ones(256, device=DEV)
-    with pytest.raises(L.CatcocError, match="k % 64"):
-        ops.quant_matmul_splitk(x1, x2, s1, s2, None, [], 1, 0, 2)
     x1 = torch.zeros((16, 2048), dtype=torch.int8, device=DEV)
     x2 = torch.zeros((2048, 256), dtype=torch.int8, device=DEV)
     with pytest.raises(L.CatcocError, match="workspace"):
