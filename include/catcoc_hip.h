@@ -318,7 +318,9 @@ CATCOC_API uint64_t catcoc_get_kslice_workspace_size(int commType, int dataType,
  * and B [k,n] (or, with transB, [n,k]: a weight matrix stored output-major), peers [keptRows, n] as fp32 added after
  * the dequantisation or, with CATCOC_FLAG_REDUCE_INT32, int32 added before it.  k in whole 64-byte steps and n in whole
  * 128-column tiles run the streaming kernels; any other k or n runs whole tiles on a one-thread-per-element kernel
- * (correct, slow, no k split).  CATCOC_OUTBOUND_STORE does not apply (explicit kept rows have no rank structure to lay
+ * (correct, slow, no k split).  At most 32 rows against B as [n,k] (k in whole 128-byte chunks, desc->splitK 0 or 1, no
+ * `checksum`) need no k split at all: one workgroup per 32 columns walks the whole k range, and such a launch neither needs
+ * nor touches the workspace, whatever this query (which does not know the layout) reports.  CATCOC_OUTBOUND_STORE does not apply (explicit kept rows have no rank structure to lay
  * tiles out by).  It stands in for SplitkMatmul (3rdparty/catlass/include/catlass/gemm/kernel/splitk_matmul.hpp:68-330)
  * in front of the dequant / reduce epilogue. */
 CATCOC_API uint64_t catcoc_get_splitk_workspace_size(const CocTilingParams *tiling, const CatcocSymmetricDesc *desc,

@@ -21,6 +21,7 @@ namespace catcoc {
 int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream);
 int launch_gemm_dma_i8(const GemmArgs &args, void *stream);
 int launch_gemm_splitk_i8(const GemmArgs &args, int rowBlocks, uint32_t tasks, void *stream);
+int launch_gemm_decode_nk_i8(const GemmArgs &args, void *stream);
 int launch_gemm_f16(const GemmArgs &args, int variant, bool edge, void *stream);
 int launch_gemm_bf16(const GemmArgs &args, int variant, bool edge, void *stream);
 int launch_gemm_dma_f16(const GemmArgs &args, void *stream);
@@ -300,6 +301,7 @@ struct SplitkPlan {
     uint32_t f, tiles, rowBlocks;
     uint64_t workspaceBytes;   // partial tiles + counters (0 when f == 1)
     bool general;              // shape outside the fast routes: gemm_general_kernel on the 128x128 grid
+    bool wholeK;               // at most 32 rows against B as [n,k]: gemm_decode_nk_kernel, no k slices, no workspace
     bool large;                // many rows: the 128x256 direct-to-LDS kernel in row-mask mode runs instead of the split-K kernel
 };
 
@@ -325,6 +327,7 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
     // shapes the two fast routes cannot take (k not in whole 64-byte steps, n not in whole 128-column tiles) run the
     // one-thread-per-element kernel on the same 128x128 grid: a correctness path, whole tiles, no workspace
     sp.general = t->k % 64 != 0 || t->n % 128 != 0;
+    sp.wholeK = false;
     const bool canLarge = !sp.general && t->m % 128 == 0 && t->n % 256 == 0 && d->keptRowBegin % 32 == 0 && d->keptRows % 32 == 0;
     const bool wantLarge = t->n0 == 256 && (t->m0 == 0 || t->m0 == 128);
     if (wantLarge && !canLarge)
@@ -400,6 +403,17 @@ int make_splitk_plan(const CocTilingParams *t, const CatcocSymmetricDesc *d, uin
         sp.workspaceBytes = f > 1 ? kCounterBlockBytes + (uint64_t)T * f * (128u * 256u * 4u) : 0;
         return 0;
     }
+    // B as [n,k] against at most 32 rows: a workgroup can own 32 columns over the whole k range and still read whole cache
+    // lines, so nothing is handed between workgroups (unless the caller asks for k slices or for per-tile checksums, which
+    // are per 128 columns)
+    sp.wholeK = transB && t->m <= 32 && t->k % 128 == 0 && d->splitK <= 1 && d->checksum == nullptr;
+    if (sp.wholeK) {
+        sp.f = 1;
+        a.splitK = 0;
+        sp.rowBlocks = 1;
+        sp.workspaceBytes = 0;
+        return 0;
+    }
     uint32_t f = d->splitK ? d->splitK : splitk_factor(t->m, t->n, t->k, cores, 128, 128, 256);
     if (f > kTiles) f = kTiles;
     if (f == 0) f = 1;
@@ -469,7 +483,7 @@ void launch_quant_splitk(void *stream, uint8_t *x1, uint8_t *x2, uint8_t *scale_
         ok();
         return;
     }
-    const int e = launch_gemm_splitk_i8(a, (int)sp.rowBlocks, sp.tiles * sp.f, stream);
+    const int e = sp.wholeK ? launch_gemm_decode_nk_i8(a, stream) : launch_gemm_splitk_i8(a, (int)sp.rowBlocks, sp.tiles * sp.f, stream);
     if (e) { fail(E_LAUNCH, "kernel launch failed: %s", hipGetErrorString((hipError_t)e)); return; }
     ok();
 }

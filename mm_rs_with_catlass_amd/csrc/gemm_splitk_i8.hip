@@ -1,4 +1,5 @@
-// Instantiates the skinny-M split-K W8A8 kernel.
+// Instantiates the skinny-M W8A8 kernels: split K, and whole K for weights stored as [n,k].
+#include "gemm_decode_nk_kernel.h"
 #include "gemm_splitk_kernel.h"
 
 namespace catcoc {
@@ -23,6 +24,17 @@ int launch_gemm_splitk_i8(const GemmArgs &args, int rowBlocks, uint32_t tasks, v
     else if (rowBlocks == 2) hipLaunchKernelGGL((gemm_splitk_kernel<2>), grid, block, 0, s, args);
     else if (pairs) hipLaunchKernelGGL((gemm_splitk_kernel<4, true>), grid, block, 0, s, args);
     else hipLaunchKernelGGL((gemm_splitk_kernel<4>), grid, block, 0, s, args);
+    return (int)hipGetLastError();
+}
+
+// At most 32 rows of A against B as [n][k] (K in whole 128-byte chunks, N in whole 32-column strips): one workgroup per strip.
+int launch_gemm_decode_nk_i8(const GemmArgs &args, void *stream)
+{
+    const dim3 grid(args.N / 32u), block(256);
+    hipStream_t s = (hipStream_t)stream;
+    if (args.M <= 8) hipLaunchKernelGGL((gemm_decode_nk_kernel<1>), grid, block, 0, s, args);
+    else if (args.M <= 16) hipLaunchKernelGGL((gemm_decode_nk_kernel<2>), grid, block, 0, s, args);
+    else hipLaunchKernelGGL((gemm_decode_nk_kernel<4>), grid, block, 0, s, args);
     return (int)hipGetLastError();
 }
 }  // namespace catcoc

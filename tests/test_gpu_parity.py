@@ -496,6 +496,48 @@ def test_quant_skinny_m_weight_layout_and_reference_reduce_order(case, mode):
     assert not ws[:65536].any()
 
 
+# (M, N, K, P, kept_begin, kept_rows, peer_row_offset, fp16 output, bias, int32 peers)
+@pytest.mark.parametrize("case", [(1, 128, 128, 1, 0, 1, 0, False, False, False), (1, 8192, 8192, 8, 0, 1, 0, False, True, False),
+                                  (8, 256, 384, 8, 5, 3, 0, False, True, True), (9, 1024, 1152, 16, 0, 9, 2, True, True, False),
+                                  (16, 8192, 8192, 8, 14, 2, 0, False, True, False), (17, 640, 2048, 4, 7, 10, 0, True, False, True),
+                                  (24, 384, 640, 16, 20, 4, 1, False, True, False), (32, 8192, 8192, 8, 0, 32, 0, False, True, True),
+                                  (31, 128, 256, 2, 30, 1, 0, True, True, False), (32, 4096, 512, 9, 8, 16, 0, False, False, True)])
+def test_quant_decode_rows_against_stored_weights_whole_k(case):
+    """At most 32 rows against B stored as [n,k]: a workgroup owns 32 columns over the whole k range (no k slices, no
+    workspace), its four waves deal the 128-byte chunks of k round-robin and start the walk at a place of their own.  One to
+    32 rows (every A-copy width), k of one chunk, of fewer chunks than waves have stages and of many, one to sixteen
+    ranks (more than one batch of eight peers), kept rows at the start, in the middle and at the end of the block, peers
+    read at a row offset, fp16 and bf16 output, with and without bias, fp32 peers and int32 peers: the accumulators of
+    every row, the kept int32 block and the output bit for bit against the oracle, twice in a row, with no workspace."""
+    _need_gpu()
+    M, N, K, P, kb, kr, pro, f16, has_bias, ri = case
+    rng = np.random.default_rng(460 + M + K)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.integers(-1000, 1000, N, dtype=np.int32) if has_bias else None
+    peers = [rng.integers(-2 ** 24, 2 ** 24, (kr, N), dtype=np.int32) if ri else rng.standard_normal((kr, N)).astype(np.float32)
+             for _ in range(P - 1)]
+    acc_want, out_want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, b, kb, kr, peers, oracle.FP16 if f16 else oracle.BF16,
+                                                            reduce_int32=ri)
+    # peers as the launch sees them: `pro` rows of filler in front of the rows that line up with the kept ones
+    staged = [np.concatenate([np.full((pro, N), 77, p.dtype), p]) for p in peers]
+    acc_dump = torch.full((M, N), -7, dtype=torch.int32, device=DEV)
+    c_accum = torch.full((kr, N), -7, dtype=torch.int32, device=DEV)
+    launch, out = ops.prepare_quant_matmul_splitk(dev(x1), dev(np.ascontiguousarray(x2.T)), dev(s1), dev(s2), dev(b) if has_bias else None,
+                                                  [dev(p) for p in staged], P, kb, kr, out_dtype=torch.float16 if f16 else torch.bfloat16,
+                                                  acc_dump=acc_dump, c_accum=c_accum, peer_row_offset=pro, trans_b=True, reduce_int32=ri)
+    for it in range(2):
+        out.zero_()
+        launch()
+        L.check()
+        torch.cuda.synchronize()
+        assert np.array_equal(acc_dump.cpu().numpy(), acc_want), "int32 accumulators differ from the oracle"
+        assert np.array_equal(c_accum.cpu().numpy(), acc_want[kb:kb + kr] + (sum(peers) if ri else 0)), "kept int32 block differs"
+        assert np.array_equal(host16(out), out_want), "kept rows differ from the oracle"
+
+
 @pytest.mark.parametrize("case", [(40, 200, 100, 4, 5, 20, False, False), (130, 264, 192, 2, 100, 30, True, False), (17, 128, 72, 8, 0, 17, False, True),
                                   (260, 136, 1000, 4, 120, 140, True, True)])
 def test_quant_explicit_kept_rows_on_odd_shapes(case):
