@@ -24,49 +24,44 @@
 
 namespace catcoc {
 
-// ACP: 1 KiB copies of A per chunk (8 rows each): 1, 2 or 4 for up to 8, 16 or 32 rows of A.  Rows of the A stage that
-// are not copied hold stale bytes; they only feed accumulator rows that are never looked at.
-template <int ACP>
-__global__ void __launch_bounds__(256, 1) gemm_decode_nk_kernel(const GemmArgs args)
-{
-    constexpr int B_STAGE = 32 * 128, A_STAGE = ACP * 1024, STAGE = B_STAGE + A_STAGE;
-    constexpr int NS = (40 * 1024) / STAGE;     // stages per wave: 8, 6 or 5, one less than that many chunks in flight
-    constexpr int CP = 4 + ACP;                 // copies per chunk
-    constexpr int WAVE_POOL = 40 * 1024;
-    static_assert(4 * WAVE_POOL <= 160 * 1024, "four rings fit the LDS of a CU");
-    static_assert((NS - 1) * CP <= 63, "the wait counter holds 63");
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * WAVE_POOL];
+// One 32 x 32 block of accumulators in MFMA layout -- acc[r] of lane (c32, h) is element (row, col) =
+// (rowBase + slot_row(r) + 4h, gcol) -- and what the epilogue does with it: bias, accumulator dump, int32 peers, kept
+// int32 block, dequantisation, fp32 peers, 16-bit store of the kept rows.  The wave that owns the block requests bias,
+// scales and the first eight peers (prefetch) long before it has the sums (finish).
+struct DecodeBlock {
+    uint32_t rowBase, rowsValid, gcol, h;
+    uint32_t kLo, kN, rel;          // kept rows of the block: [kLo, kLo + kN) counted from rowBase
+    uint32_t peerPitch, peerBase;
+    int peerRange;
+    int bv;
+    float sN, sMrow;
+    float pv[8][16];
+    static constexpr uint32_t OUT_OF_RANGE = 0x7fffffffu;   // a buffer load at this offset touches no memory and reads zero
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // (wave-uniform by construction; this tells the compiler)
-    const int c32 = lane & 31, h = lane >> 5;
-    const uint32_t M = args.M, N = args.N, K = args.K;
-    const uint32_t col0 = blockIdx.x * 32u;
-    if (col0 >= N) return;
-    const uint32_t nChunks = K / 128u;
-    const uint32_t mine = nChunks > (uint32_t)w ? (nChunks - (uint32_t)w + 3u) / 4u : 0u;   // chunks w, w + 4, ...
-    const int64_t lda = args.lda, ldb = args.ldb;
-    unsigned char *ring = smem + w * WAVE_POOL;
-    const uint32_t ring0 = (uint32_t)(uintptr_t)(CATCOC_LDS unsigned char *)ring;
+    static __device__ __forceinline__ uint32_t slot_row(int r) { return (uint32_t)((r >> 2) * 8 + (r & 3)); }
+    __device__ __forceinline__ bool slot_active(int r) const { return slot_row(r) < kLo + kN && slot_row(r) + 4u >= kLo; }   // wave-uniform
+    __device__ __forceinline__ bool lane_kept(int r) const { return slot_row(r) + rel < kN; }
 
-    // ---- the epilogue's operands, requested first (wave 0 only) -----------------------------------------------------
-    // acc[r] is element (row, col) = (slot_row(r) + 4h, col0 + c32) of the 32 x 32 block
-    const uint32_t gcol = col0 + c32;
-    const uint32_t keptEnd = args.keptBegin + args.keptRows;
-    const uint32_t rowsValid = umin(32u, M);
-    auto slot_row = [](int r) { return (uint32_t)((r >> 2) * 8 + (r & 3)); };
-    const uint32_t kLo = umin(args.keptBegin, rowsValid), kHi = umin(keptEnd, rowsValid);   // kept rows of the block: [kLo, kHi)
-    const uint32_t kN = kHi > kLo ? kHi - kLo : 0u;
-    const uint32_t rel = 4u * h - kLo;
-    auto slot_active = [&](int r) { return slot_row(r) < kLo + kN && slot_row(r) + 4u >= kLo; };   // wave-uniform
-    auto lane_kept = [&](int r) { return slot_row(r) + rel < kN; };
-    const uint64_t peerBytes = (uint64_t)(args.peerRowOffset + args.keptRows) * args.peerLd * 4;
-    const int peerRange = peerBytes > 0x7fffffffull ? 0x7fffffff : (int)peerBytes;
-    const uint32_t peerPitch = (uint32_t)args.peerLd * 4u;
-    const uint32_t peerBase = ((uint32_t)args.peerRowOffset + 4u * h - args.keptBegin) * peerPitch + gcol * 4u;   // + slot_row * pitch
-    constexpr uint32_t OUT_OF_RANGE = 0x7fffffffu;   // a buffer load at this offset touches no memory and reads zero
-    auto fetch_peers = [&](uint32_t p0, float (&pv)[8][16]) {
+    __device__ __forceinline__ void init(const GemmArgs &args, uint32_t rowBase_, uint32_t gcol_, uint32_t h_)
+    {
+        rowBase = rowBase_; gcol = gcol_; h = h_;
+        rowsValid = umin(32u, args.M - rowBase);
+        const uint32_t keptEnd = args.keptBegin + args.keptRows;
+        const uint32_t lo = args.keptBegin > rowBase ? args.keptBegin - rowBase : 0u;
+        const uint32_t hi = keptEnd > rowBase ? keptEnd - rowBase : 0u;
+        kLo = umin(lo, rowsValid);
+        const uint32_t kHi = umin(hi, rowsValid);
+        kN = kHi > kLo ? kHi - kLo : 0u;
+        rel = 4u * h - kLo;
+        const uint64_t peerBytes = (uint64_t)(args.peerRowOffset + args.keptRows) * args.peerLd * 4;
+        peerRange = peerBytes > 0x7fffffffull ? 0x7fffffff : (int)peerBytes;
+        peerPitch = (uint32_t)args.peerLd * 4u;
+        // + slot_row * pitch; only kept lanes use it, so the wrap of rows before the kept range never reaches memory
+        peerBase = ((uint32_t)args.peerRowOffset + rowBase + 4u * h - args.keptBegin) * peerPitch + gcol * 4u;
+        bv = 0; sN = 0.f; sMrow = 0.f;
+    }
+    __device__ __forceinline__ void fetch_peers(const GemmArgs &args, uint32_t p0)
+    {
         __amdgpu_buffer_rsrc_t prs[8];
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
@@ -85,16 +80,119 @@ __global__ void __launch_bounds__(256, 1) gemm_decode_nk_kernel(const GemmArgs a
                 for (int q = 0; q < 8; ++q) pv[q][r] = 0.0f;
             }
         }
-    };
-    int bv = 0;
-    float sN = 0.f, sMrow = 0.f;
-    float pv0[8][16];
-    if (w == 0) {
+    }
+    __device__ __forceinline__ void prefetch(const GemmArgs &args, uint32_t c32)
+    {
         bv = args.bias ? args.bias[gcol] : 0;
         sN = args.scaleN[gcol];
-        sMrow = (uint32_t)c32 < rowsValid ? args.scaleM[c32] : 0.0f;   // lane l fetches row l; picked per slot in the epilogue
-        fetch_peers(0, pv0);
+        sMrow = c32 < rowsValid ? args.scaleM[rowBase + c32] : 0.0f;   // lane l fetches row l; picked per slot in finish()
+        fetch_peers(args, 0);
     }
+    __device__ __forceinline__ void finish(const GemmArgs &args, const v16i &acc)
+    {
+        const uint32_t N = args.N;
+        const bool redI32 = (args.flags & GF_REDUCE_INT32) != 0;
+        int iv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) iv[r] = acc[r] + bv;
+        if (args.accDump) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (slot_row(r) + 4u * h < rowsValid) ((int32_t *)args.accDump)[(size_t)(rowBase + slot_row(r) + 4u * h) * N + gcol] = iv[r];
+        }
+        if (kN == 0) return;
+        if (redI32) {   // int32 peers join the accumulators before the dequantisation (quant_matmul_reduce_scatter.hpp:285-351)
+            for (uint32_t p0 = 0; p0 < args.nPeers; p0 += 8) {
+                if (p0 != 0) fetch_peers(args, p0);
+#pragma unroll
+                for (int q = 0; q < 8; ++q)
+                    if (p0 + q < args.nPeers) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) iv[r] += f2i(pv[q][r]);   // (the loads carry bit patterns)
+                    }
+            }
+        }
+        // signed row arithmetic below: the block starts at rowBase, the kept rows anywhere in it (only kept lanes dereference)
+        const int64_t keptRow0 = (int64_t)rowBase + 4 * (int64_t)h - (int64_t)args.keptBegin;   // + slot_row
+        if (args.cAccum) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (lane_kept(r)) args.cAccum[(keptRow0 + slot_row(r)) * (int64_t)N + gcol] = iv[r];
+        }
+        float v[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = __fmul_rn(__fmul_rn((float)iv[r], sN), __shfl(sMrow, slot_row(r) + 4 * h, 64));
+        for (uint32_t p0 = 0; p0 < (redI32 ? 0u : args.nPeers); p0 += 8) {
+            if (p0 != 0) fetch_peers(args, p0);
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+                if (p0 + q < args.nPeers) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) v[r] = __fadd_rn(v[r], pv[q][r]);
+                }
+        }
+        unsigned short *drow = (unsigned short *)args.d + keptRow0 * args.ldd + gcol;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            if (lane_kept(r)) drow[(int64_t)slot_row(r) * args.ldd] = (unsigned short)f32_to_out16(v[r], args.outDtype);
+    }
+};
+
+// At most n whole chunks of CP copies each (the youngest) may still be in flight.
+template <int CP, int NMAX>
+__device__ __forceinline__ void wait_copies_but(uint32_t n)
+{
+    static_assert(NMAX * CP <= 63 && NMAX <= 15, "the wait counter holds 63");
+    if (n >= (uint32_t)NMAX) { CATCOC_WAIT_VMCNT(NMAX * CP); return; }   // the steady state
+    switch (n) {
+        case 0: CATCOC_WAIT_VMCNT(0); break;
+        case 1: CATCOC_WAIT_VMCNT(1 * CP); break;
+        case 2: CATCOC_WAIT_VMCNT(2 * CP); break;
+        case 3: CATCOC_WAIT_VMCNT(3 * CP); break;
+        case 4: CATCOC_WAIT_VMCNT(4 * CP); break;
+        case 5: CATCOC_WAIT_VMCNT(5 * CP); break;
+        case 6: CATCOC_WAIT_VMCNT(6 * CP); break;
+        case 7: CATCOC_WAIT_VMCNT(7 * CP); break;
+        case 8: CATCOC_WAIT_VMCNT(8 * CP); break;
+        case 9: CATCOC_WAIT_VMCNT(9 * CP); break;
+        case 10: CATCOC_WAIT_VMCNT(10 * CP); break;
+        case 11: CATCOC_WAIT_VMCNT(11 * CP); break;
+        case 12: CATCOC_WAIT_VMCNT(12 * CP); break;
+        case 13: CATCOC_WAIT_VMCNT(13 * CP); break;
+        default: CATCOC_WAIT_VMCNT(14 * CP); break;
+    }
+}
+
+// ACP: 1 KiB copies of A per chunk (8 rows each): 1, 2 or 4 for up to 8, 16 or 32 rows of A.  Rows of the A stage that
+// are not copied hold stale bytes; they only feed accumulator rows that are never looked at.
+template <int ACP>
+__global__ void __launch_bounds__(256, 1) gemm_decode_nk_kernel(const GemmArgs args)
+{
+    constexpr int B_STAGE = 32 * 128, A_STAGE = ACP * 1024, STAGE = B_STAGE + A_STAGE;
+    constexpr int NS = (40 * 1024) / STAGE;     // stages per wave: 8, 6 or 5, one less than that many chunks in flight
+    constexpr int CP = 4 + ACP;                 // copies per chunk
+    constexpr int WAVE_POOL = 40 * 1024;
+    static_assert(4 * WAVE_POOL <= 160 * 1024, "four rings fit the LDS of a CU");
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[4 * WAVE_POOL];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // (wave-uniform by construction; this tells the compiler)
+    const int c32 = lane & 31, h = lane >> 5;
+    const uint32_t M = args.M, N = args.N, K = args.K;
+    const uint32_t col0 = blockIdx.x * 32u;
+    if (col0 >= N) return;
+    const uint32_t nChunks = K / 128u;
+    const uint32_t mine = nChunks > (uint32_t)w ? (nChunks - (uint32_t)w + 3u) / 4u : 0u;   // chunks w, w + 4, ...
+    const int64_t lda = args.lda, ldb = args.ldb;
+    unsigned char *ring = smem + w * WAVE_POOL;
+    const uint32_t ring0 = (uint32_t)(uintptr_t)(CATCOC_LDS unsigned char *)ring;
+
+    // ---- the epilogue's operands, requested first (wave 0 only): older than every copy, they cost the ring's waits nothing
+    DecodeBlock blk;
+    blk.init(args, 0u, col0 + c32, h);
+    const uint32_t rowsValid = blk.rowsValid;
+    if (w == 0) blk.prefetch(args, c32);
 
     // ---- the stream ---------------------------------------------------------------------------------------------------
     // Stage layout: rows of 128 bytes, 16-byte chunk c of row r at slot c ^ ((r >> 1) & 7); copy j covers rows 8j .. 8j+7
@@ -137,17 +235,6 @@ __global__ void __launch_bounds__(256, 1) gemm_decode_nk_kernel(const GemmArgs a
             for (int j = 0; j < ACP; ++j) gA[j] -= back;
         }
     };
-    auto wait_chunks = [&](uint32_t n) {   // at most n whole chunks of copies (the youngest) outstanding; n <= NS - 2
-        if (n >= (uint32_t)(NS - 2)) { CATCOC_WAIT_VMCNT((NS - 2) * CP); return; }   // the steady state
-        switch (n) {
-            case 0: CATCOC_WAIT_VMCNT(0); break;
-            case 1: CATCOC_WAIT_VMCNT(1 * CP); break;
-            case 2: CATCOC_WAIT_VMCNT(2 * CP); break;
-            case 3: CATCOC_WAIT_VMCNT(3 * CP); break;
-            case 4: CATCOC_WAIT_VMCNT(4 * CP); break;
-            default: CATCOC_WAIT_VMCNT(5 * CP); break;
-        }
-    };
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0;
@@ -157,7 +244,7 @@ __global__ void __launch_bounds__(256, 1) gemm_decode_nk_kernel(const GemmArgs a
     uint32_t issued = 0;
     for (; issued < umin(mine, (uint32_t)(NS - 1)); ++issued) issue(issued);
     for (uint32_t i = 0; i < mine; ++i) {
-        wait_chunks(issued - (i + 1u));
+        wait_copies_but<CP, NS - 2>(issued - (i + 1u));
         asm volatile("" ::: "memory");
         const unsigned char *sb = ring + (i % NS) * STAGE, *sa = sb + B_STAGE;
         v4i bf[4], af[4];
@@ -175,7 +262,7 @@ __global__ void __launch_bounds__(256, 1) gemm_decode_nk_kernel(const GemmArgs a
         for (int kk = 0; kk < 4; ++kk) acc = mfma32<DT_I8>(af[kk], bf[kk], acc);
     }
 
-    // ---- the four partial blocks meet in LDS; wave 0 adds them ----------------------------------------------------------
+    // ---- the four partial blocks meet in LDS; wave 0 adds them and finishes the rows that exist --------------------------
     CATCOC_WAIT_VMCNT(0);
     __syncthreads();   // every wave has left its ring
     int *meet = (int *)smem;   // [3][16][64]
@@ -189,51 +276,7 @@ __global__ void __launch_bounds__(256, 1) gemm_decode_nk_kernel(const GemmArgs a
     for (int o = 0; o < 3; ++o)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] += meet[(o * 16 + r) * 64 + lane];
-
-    // ---- epilogue on the rows that exist ------------------------------------------------------------------------------
-    const bool redI32 = (args.flags & GF_REDUCE_INT32) != 0;
-    int iv[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) iv[r] = acc[r] + bv;
-    if (args.accDump) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-            if (slot_row(r) + 4u * h < rowsValid) ((int32_t *)args.accDump)[(size_t)(slot_row(r) + 4u * h) * N + gcol] = iv[r];
-    }
-    if (kN == 0) return;
-    if (redI32) {   // int32 peers join the accumulators before the dequantisation (quant_matmul_reduce_scatter.hpp:285-351)
-        for (uint32_t p0 = 0; p0 < args.nPeers; p0 += 8) {
-            if (p0 != 0) fetch_peers(p0, pv0);
-#pragma unroll
-            for (int q = 0; q < 8; ++q)
-                if (p0 + q < args.nPeers) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) iv[r] += f2i(pv0[q][r]);   // (the loads carry bit patterns)
-                }
-        }
-    }
-    if (args.cAccum) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-            if (lane_kept(r)) args.cAccum[(size_t)(slot_row(r) + 4u * h - args.keptBegin) * N + gcol] = iv[r];
-    }
-    float v[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) v[r] = __fmul_rn(__fmul_rn((float)iv[r], sN), __shfl(sMrow, slot_row(r) + 4 * h, 64));
-    for (uint32_t p0 = 0; p0 < (redI32 ? 0u : args.nPeers); p0 += 8) {
-        if (p0 != 0) fetch_peers(p0, pv0);
-#pragma unroll
-        for (int q = 0; q < 8; ++q)
-            if (p0 + q < args.nPeers) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) v[r] = __fadd_rn(v[r], pv0[q][r]);
-            }
-    }
-    // signed: the block starts at row 0, the kept rows anywhere in it (only kept lanes dereference)
-    unsigned short *drow = (unsigned short *)args.d + ((int64_t)(4u * h) - (int64_t)args.keptBegin) * args.ldd + gcol;
-#pragma unroll
-    for (int r = 0; r < 16; ++r)
-        if (lane_kept(r)) drow[(int64_t)slot_row(r) * args.ldd] = (unsigned short)f32_to_out16(v[r], args.outDtype);
+    blk.finish(args, acc);
 }
 
 }  // namespace catcoc

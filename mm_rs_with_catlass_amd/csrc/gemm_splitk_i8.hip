@@ -32,6 +32,7 @@ int launch_gemm_decode_nk_i8(const GemmArgs &args, void *stream)
 {
     const dim3 grid(args.N / 32u), block(256);
     hipStream_t s = (hipStream_t)stream;
+    if (args.M > 32u || args.K % 128u != 0 || args.N % 32u != 0 || args.K == 0) return (int)hipErrorInvalidValue;
     if (args.M <= 8) hipLaunchKernelGGL((gemm_decode_nk_kernel<1>), grid, block, 0, s, args);
     else if (args.M <= 16) hipLaunchKernelGGL((gemm_decode_nk_kernel<2>), grid, block, 0, s, args);
     else hipLaunchKernelGGL((gemm_decode_nk_kernel<4>), grid, block, 0, s, args);

@@ -501,14 +501,19 @@ def test_quant_skinny_m_weight_layout_and_reference_reduce_order(case, mode):
                                   (8, 256, 384, 8, 5, 3, 0, False, True, True), (9, 1024, 1152, 16, 0, 9, 2, True, True, False),
                                   (16, 8192, 8192, 8, 14, 2, 0, False, True, False), (17, 640, 2048, 4, 7, 10, 0, True, False, True),
                                   (24, 384, 640, 16, 20, 4, 1, False, True, False), (32, 8192, 8192, 8, 0, 32, 0, False, True, True),
-                                  (31, 128, 256, 2, 30, 1, 0, True, True, False), (32, 4096, 512, 9, 8, 16, 0, False, False, True)])
-def test_quant_decode_rows_against_stored_weights_whole_k(case):
-    """At most 32 rows against B stored as [n,k]: a workgroup owns 32 columns over the whole k range (no k slices, no
-    workspace), its four waves deal the 128-byte chunks of k round-robin and start the walk at a place of their own.  One to
-    32 rows (every A-copy width), k of one chunk, of fewer chunks than waves have stages and of many, one to sixteen
-    ranks (more than one batch of eight peers), kept rows at the start, in the middle and at the end of the block, peers
-    read at a row offset, fp16 and bf16 output, with and without bias, fp32 peers and int32 peers: the accumulators of
-    every row, the kept int32 block and the output bit for bit against the oracle, twice in a row, with no workspace."""
+                                  (31, 128, 256, 2, 30, 1, 0, True, True, False), (32, 4096, 512, 9, 8, 16, 0, False, False, True),
+                                  (33, 128, 256, 2, 31, 2, 0, False, True, False), (64, 8192, 8192, 8, 8, 8, 0, False, True, False),
+                                  (100, 640, 1152, 4, 20, 70, 3, True, True, True), (128, 8192, 8192, 8, 112, 16, 0, False, True, False),
+                                  (128, 256, 512, 16, 0, 128, 0, False, False, True), (96, 384, 384, 3, 60, 36, 0, True, True, False),
+                                  (65, 128, 128, 1, 64, 1, 0, False, True, False)])
+def test_quant_decode_rows_against_stored_weights(case):
+    """B stored as [n,k].  At most 32 rows: a workgroup owns 32 columns over the whole k range (no k slices, no workspace),
+    its four waves deal the 128-byte chunks of k round-robin and start the walk at a place of their own.  One to 32 rows
+    (every A-copy width), k of one chunk, of fewer chunks than waves have stages and of many, one to sixteen ranks (more
+    than one batch of eight peers), kept rows at the start, in the middle and at the end of the block, peers read at a row
+    offset, fp16 and bf16 output, with and without bias, fp32 peers and int32 peers.  33 to 128 rows: the same options on
+    the split-K kernel (with its workspace), kept rows across 32-row blocks and a last block of one row.  The accumulators
+    of every row, the kept int32 block and the output bit for bit against the oracle, twice in a row."""
     _need_gpu()
     M, N, K, P, kb, kr, pro, f16, has_bias, ri = case
     rng = np.random.default_rng(460 + M + K)
@@ -525,9 +530,14 @@ def test_quant_decode_rows_against_stored_weights_whole_k(case):
     staged = [np.concatenate([np.full((pro, N), 77, p.dtype), p]) for p in peers]
     acc_dump = torch.full((M, N), -7, dtype=torch.int32, device=DEV)
     c_accum = torch.full((kr, N), -7, dtype=torch.int32, device=DEV)
+    ws = None
+    if M > 32:
+        need, fac, tiles = ops.splitk_plan(M, K, N, P, kb, kr)
+        ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=DEV)
     launch, out = ops.prepare_quant_matmul_splitk(dev(x1), dev(np.ascontiguousarray(x2.T)), dev(s1), dev(s2), dev(b) if has_bias else None,
                                                   [dev(p) for p in staged], P, kb, kr, out_dtype=torch.float16 if f16 else torch.bfloat16,
-                                                  acc_dump=acc_dump, c_accum=c_accum, peer_row_offset=pro, trans_b=True, reduce_int32=ri)
+                                                  acc_dump=acc_dump, c_accum=c_accum, peer_row_offset=pro, trans_b=True, reduce_int32=ri,
+                                                  workspace=ws)
     for it in range(2):
         out.zero_()
         launch()
