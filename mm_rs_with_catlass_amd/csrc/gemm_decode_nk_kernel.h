@@ -180,7 +180,11 @@ __global__ void __launch_bounds__(256, 1) gemm_decode_nk_kernel(const GemmArgs a
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // (wave-uniform by construction; this tells the compiler)
     const int c32 = lane & 31, h = lane >> 5;
     const uint32_t M = args.M, N = args.N, K = args.K;
-    const uint32_t col0 = blockIdx.x * 32u;
+    // consecutive workgroups go round-robin to the eight XCDs: XCD x takes strips x * (strips / 8) onwards, neighbours in
+    // memory, when the strips deal out evenly
+    const uint32_t strips = gridDim.x;
+    const uint32_t strip = strips % 8u == 0 ? (blockIdx.x & 7u) * (strips / 8u) + (blockIdx.x >> 3) : blockIdx.x;
+    const uint32_t col0 = strip * 32u;
     if (col0 >= N) return;
     const uint32_t nChunks = K / 128u;
     const uint32_t mine = nChunks > (uint32_t)w ? (nChunks - (uint32_t)w + 3u) / 4u : 0u;   // chunks w, w + 4, ...
