@@ -1560,6 +1560,8 @@ def test_launches_replay_from_a_hip_graph():
     assert fac == 4
     ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
     small, out_small = ops.prepare_quant_matmul_splitk(xs, w, ss, s2, None, pk, P, 4, 2, split_k=4, workspace=ws)
+    # the same rows against the weights stored as [n,k]: whole k per column strip, no workspace at all
+    strips, out_strips = ops.prepare_quant_matmul_splitk(xs, w.t().contiguous(), ss, s2, None, pk, P, 4, 2, trans_b=True)
     # a launch of 512 tiles with split kept tiles, whose waiting tiles run as halves: their checksum halves meet through
     # the counter block of a workspace and clear it again
     xh = torch.randint(-127, 128, (4096, 128), dtype=torch.int8, device=DEV, generator=g)
@@ -1585,9 +1587,10 @@ def test_launches_replay_from_a_hip_graph():
     def pipe():
         ops.pipelined_quant_matmul_reduce_scatter(x1, x2, s1, s2, None, ipeers, 1, P, obp, c_accum=cacc_pipe, tiling=tp, comm_stream=comm,
                                                   block_num=8, out=out_pipe, plan=plan)
-    big(); small(); halves(); pipe(); L.check()
+    big(); small(); strips(); halves(); pipe(); L.check()
     torch.cuda.synchronize()
     want_big, want_small, want_halves, want_cs = out_big.clone(), out_small.clone(), out_halves.clone(), csh.clone()
+    assert torch.equal(out_strips, want_small), "the two weight layouts give the same rows"
     want_pipe, want_cacc = out_pipe.clone(), cacc_pipe.clone()
     fused = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, ipeers, 1, P, reduce_int32=True)
     assert torch.equal(fused.view(torch.int16), want_pipe.view(torch.int16))
@@ -1597,21 +1600,24 @@ def test_launches_replay_from_a_hip_graph():
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
-        big(); small(); halves(); pipe()     # warm the side stream before capture
+        big(); small(); strips(); halves(); pipe()     # warm the side stream before capture
         torch.cuda.synchronize()
         with torch.cuda.graph(graph, stream=side):
             out_big.zero_()
             out_small.zero_()
+            out_strips.zero_()
             out_halves.zero_()
             csh.zero_()
             big()
             small()
+            strips()
             halves()
             pipe()
     L.check()
     for _ in range(3):
         out_big.fill_(1.0)                   # eager work between the replays
         out_small.fill_(1.0)
+        out_strips.fill_(1.0)
         out_halves.fill_(1.0)
         out_pipe.fill_(1.0)
         cacc_pipe.fill_(3)
@@ -1619,7 +1625,7 @@ def test_launches_replay_from_a_hip_graph():
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(out_big, want_big) and torch.equal(out_small, want_small)
+        assert torch.equal(out_big, want_big) and torch.equal(out_small, want_small) and torch.equal(out_strips, want_small)
         assert torch.equal(out_halves, want_halves) and torch.equal(csh, want_cs)
         assert torch.equal(out_pipe, want_pipe) and torch.equal(cacc_pipe, want_cacc)
         assert not ws[:65536].any(), "tile counters were not re-armed"
