@@ -6,23 +6,25 @@ namespace catcoc {
 // rowBlocks: 32-row blocks of A a tile stages (1, 2 or 4); grid = tiles x k slices.
 int launch_gemm_splitk_i8(const GemmArgs &args, int rowBlocks, uint32_t tasks, void *stream)
 {
-    const dim3 grid(tasks), block(256);
+    const dim3 grid(tasks), block(256), block8(512);
     // k slices are whole 256-byte k tiles except the last one, which takes what is left of K: with K a multiple of 128
-    // every slice is a whole number of pairs of 64-byte steps, and A can be fetched as whole 128-byte lines
+    // every slice is a whole number of pairs of 64-byte steps, and A can be fetched as whole 128-byte lines.  128-row
+    // tiles on pairs run eight waves, one of each SIMD's two per step of a pair (measured against four waves, launches
+    // alternating: 128 rows 29.1 -> 27.4 us, 96 rows 29.2 -> 27.0; 64-row tiles do not gain, 22.2 -> 22.4).
     const bool pairs = args.K % 128u == 0;
     hipStream_t s = (hipStream_t)stream;
     if (args.transB) {   // B as [n][k]
         if (rowBlocks == 1) hipLaunchKernelGGL((gemm_splitk_kernel<1, false, true>), grid, block, 0, s, args);
         else if (rowBlocks == 2 && pairs) hipLaunchKernelGGL((gemm_splitk_kernel<2, true, true>), grid, block, 0, s, args);
         else if (rowBlocks == 2) hipLaunchKernelGGL((gemm_splitk_kernel<2, false, true>), grid, block, 0, s, args);
-        else if (pairs) hipLaunchKernelGGL((gemm_splitk_kernel<4, true, true>), grid, block, 0, s, args);
+        else if (pairs) hipLaunchKernelGGL((gemm_splitk_kernel<4, true, true, true>), grid, block8, 0, s, args);
         else hipLaunchKernelGGL((gemm_splitk_kernel<4, false, true>), grid, block, 0, s, args);
         return (int)hipGetLastError();
     }
     if (rowBlocks == 1) hipLaunchKernelGGL((gemm_splitk_kernel<1>), grid, block, 0, s, args);
     else if (rowBlocks == 2 && pairs) hipLaunchKernelGGL((gemm_splitk_kernel<2, true>), grid, block, 0, s, args);
     else if (rowBlocks == 2) hipLaunchKernelGGL((gemm_splitk_kernel<2>), grid, block, 0, s, args);
-    else if (pairs) hipLaunchKernelGGL((gemm_splitk_kernel<4, true>), grid, block, 0, s, args);
+    else if (pairs) hipLaunchKernelGGL((gemm_splitk_kernel<4, true, false, true>), grid, block8, 0, s, args);
     else hipLaunchKernelGGL((gemm_splitk_kernel<4>), grid, block, 0, s, args);
     return (int)hipGetLastError();
 }

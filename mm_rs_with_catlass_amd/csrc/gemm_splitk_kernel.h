@@ -33,11 +33,17 @@ namespace catcoc {
 // TB: B is given as [n][k] (k contiguous, the layout of a stored weight matrix): a step's B stage is then 128 rows of 64
 // bytes of k, copied and read exactly like A's (plain 16-byte fragment reads, no transposing reads).  A line of B is
 // asked for in two halves one step apart; the second finds it in L2, so these copies carry no streaming hint.
-template <int MBW, bool AP = false, bool TB = false>
-__global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args)
+// KP: eight waves, two per SIMD: waves 4-7 own the same columns as waves 0-3 and take the second step of every pair
+// (accumulators of their own, added to the others' through LDS after the loop).  A wave alone on its SIMD reads its
+// fragments, multiplies, waits at the barrier and issues copies one after the other, and the four waves do so in lockstep,
+// so LDS, matrix pipe and copy path take turns; with a second wave per SIMD on the other step they overlap.
+template <int MBW, bool AP = false, bool TB = false, bool KP = false>
+__global__ void __launch_bounds__(KP ? 512 : 256, 1) gemm_splitk_kernel(const GemmArgs args)
 {
     static_assert(!AP || MBW >= 2, "pairs of steps are the groups of the 64- and 128-row tiles");
-    constexpr int NW = 4;
+    static_assert(!KP || AP, "the step-parity split works on pairs of steps");
+    constexpr int NW = KP ? 8 : 4;             // waves that issue copies
+    constexpr int PB = KP ? 4 : 8;             // peers whose values a wave holds at a time
     constexpr int G = (MBW == 1) ? 4 : 2;      // k steps per barrier
     constexpr int NS = (MBW == 1) ? 12 : 8;    // LDS stages (a multiple of G, at least 2G)
     constexpr int ROWS = 32 * MBW;
@@ -45,13 +51,16 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     constexpr int B_STAGE = 64 * 128;
     constexpr int STAGE = A_STAGE + B_STAGE;
     constexpr int A_CP = (MBW >= 2) ? MBW / 2 : 1;   // A copies per wave per step (MBW 1: waves 2,3 repeat 0,1)
-    constexpr int B_CP = 2;
+    constexpr int B_CP = 8 / NW;
+    constexpr int PAIR_CP = MBW * 4 / NW + 2 * B_CP;   // pair instantiations: copies per wave per pair of steps
     constexpr int STEP_CP = A_CP + B_CP;
     __shared__ __attribute__((aligned(1024))) unsigned char smem[NS * STAGE];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int w = tid >> 6;
+    const int wc = tid >> 6;                   // wave of the workgroup: which copies it issues
+    const int w = wc & 3;                      // its 32 columns of the tile
+    const int kp = KP ? wc >> 2 : 0;           // its step of every pair
     const int c32 = lane & 31, h = lane >> 5;
 
     const uint32_t M = args.M, N = args.N, K = args.K, f = args.splitK;
@@ -74,7 +83,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     auto copy_b = [&](const unsigned char *Bgk, unsigned char *sb) {
 #pragma unroll
         for (int jj = 0; jj < B_CP; ++jj) {
-            const int j = w + NW * jj;
+            const int j = wc + NW * jj;
             if constexpr (TB) {
                 const uint32_t lrow = 16 * j + (lane >> 2);
                 dma16(Bgk + (size_t)lrow * ldb + (((lane & 3) ^ ((lane >> 4) & 3)) * 16), sb + j * 1024);
@@ -112,8 +121,8 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         const uint32_t kt = step + rot < nsteps ? step + rot : step + rot - nsteps;
         const unsigned char *Agk = Ag + (size_t)kt * 64;
 #pragma unroll
-        for (int jj = 0; jj < MBW; ++jj) {
-            const int j = w + NW * jj;
+        for (int jj = 0; jj < MBW * 4 / NW; ++jj) {
+            const int j = wc + NW * jj;
             const uint32_t lrow = 8 * j + (lane >> 3);
             const uint32_t srow = umin(lrow, rowsValid - 1u);
             dma16(Agk + (size_t)srow * lda + (((lane & 7) ^ ((lrow >> 1) & 7)) * 16), sp + j * 1024);
@@ -167,11 +176,12 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     };
     auto slot_active = [&](const KeptRows &k, int r) { return slot_row(r) < k.lo + k.n && slot_row(r) + 4u >= k.lo; };   // uniform
     auto lane_kept = [&](const KeptRows &k, int r) { return slot_row(r) + k.rel < k.n; };
-    // eight peers of one block, slot by slot: one uniform test, then eight loads back to back
-    auto fetch_peers = [&](const KeptRows &k, uint32_t p0, float (&pv)[8][16]) {
-        __amdgpu_buffer_rsrc_t prs[8];   // a peer that does not exist gets an empty range
+    // PB peers of one block (eight; four where two waves share a SIMD's registers), slot by slot: one uniform test, then
+    // the loads back to back
+    auto fetch_peers = [&](const KeptRows &k, uint32_t p0, float (&pv)[PB][16]) {
+        __amdgpu_buffer_rsrc_t prs[PB];   // a peer that does not exist gets an empty range
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
+        for (int q = 0; q < PB; ++q) {
             const bool use = p0 + q < args.nPeers && k.n != 0;
             prs[q] = __builtin_amdgcn_make_buffer_rsrc((void *)args.peers[use ? p0 + q : 0], 0, use ? peerRange : 0, 0x00020000);
         }
@@ -180,11 +190,11 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
             if (k.n != 0 && slot_active(k, r)) {
                 const uint32_t off = lane_kept(k, r) ? k.base + slot_row(r) * peerPitch : OUT_OF_RANGE;
 #pragma unroll
-                for (int q = 0; q < 8; ++q)
+                for (int q = 0; q < PB; ++q)
                     pv[q][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(prs[q], off, 0, 2 /* streaming */));
             } else {
 #pragma unroll
-                for (int q = 0; q < 8; ++q) pv[q][r] = 0.0f;
+                for (int q = 0; q < PB; ++q) pv[q][r] = 0.0f;
             }
         }
     };
@@ -195,7 +205,7 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     int bv;
     float sN;
     float sMrow[MBW];
-    float pv0[8][16];
+    float pv0[PB][16];
     auto request_epilogue_operands = [&]() {
         bv = args.bias ? args.bias[gcol] : 0;
         sN = args.scaleN[gcol];
@@ -228,6 +238,16 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     uint32_t issued = 0;
     while (issued < ahead) issue_more(issued);
     auto wait_steps_in_flight = [&](uint32_t n) {
+        if constexpr (AP) {   // whole pairs
+            switch (n / 2) {
+                case 0: CATCOC_WAIT_VMCNT(0); break;
+                case 1: CATCOC_WAIT_VMCNT(1 * PAIR_CP); break;
+                case 2: CATCOC_WAIT_VMCNT(2 * PAIR_CP); break;
+                case 3: CATCOC_WAIT_VMCNT(3 * PAIR_CP); break;
+                default: CATCOC_WAIT_VMCNT(4 * PAIR_CP); break;
+            }
+            return;
+        }
         switch (n) {
             case 0: CATCOC_WAIT_VMCNT(0); break;
             case 1: CATCOC_WAIT_VMCNT(1 * STEP_CP); break;
@@ -249,36 +269,38 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         while (issued < nsteps && issued < s + NS) issue_more(issued);
         // all fragment reads of the group first, then the MFMAs: one LDS round trip per group (left to itself the
         // compiler reuses two fragment registers and serialises them)
-        v4i bf[GG][2], af[GG][2][MBW];
+        constexpr int GJ = KP ? 1 : GG;   // steps of the group this wave multiplies (KP: the one of its parity)
+        v4i bf[GJ][2], af[GJ][2][MBW];
 #pragma unroll
-        for (int j = 0; j < GG; ++j) {
+        for (int jj = 0; jj < GJ; ++jj) {
+            const int j = KP ? kp : jj;
             // (AP: the group's area starts at the stage of its first step: the pair of A, then B of step j)
             const unsigned char *sa = AP ? smem + (s % NS) * STAGE : smem + ((s + j) % NS) * STAGE;
             const unsigned char *sb = AP ? sa + 2 * A_STAGE + j * B_STAGE : sa + A_STAGE;
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
                 if constexpr (TB) {
-                    bf[j][kk] = *(const v4i *)(sb + bt_lds + (((2 * kk + h) ^ a_sw) * 16));
+                    bf[jj][kk] = *(const v4i *)(sb + bt_lds + (((2 * kk + h) ^ a_sw) * 16));
                 } else {
                     const unsigned char *p = sb + b_lds + kk * 32 * 128;
                     const v2i t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)p);
                     const v2i t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((CATCOC_LDS v2i *)(p + 8 * 128));
-                    bf[j][kk] = v4i{t0.x, t0.y, t1.x, t1.y};
+                    bf[jj][kk] = v4i{t0.x, t0.y, t1.x, t1.y};
                 }
 #pragma unroll
                 for (int mb = 0; mb < MBW; ++mb) {
-                    if constexpr (AP) af[j][kk][mb] = *(const v4i *)(sa + ap_lds + mb * 32 * 128 + (((4 * j + 2 * kk + h) ^ ap_sw) * 16));
-                    else af[j][kk][mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
+                    if constexpr (AP) af[jj][kk][mb] = *(const v4i *)(sa + ap_lds + mb * 32 * 128 + (((4 * j + 2 * kk + h) ^ ap_sw) * 16));
+                    else af[jj][kk][mb] = *(const v4i *)(sa + a_lds + mb * 32 * 64 + (((2 * kk + h) ^ a_sw) * 16));
                 }
             }
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < GG; ++j)
+        for (int jj = 0; jj < GJ; ++jj)
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-                for (int mb = 0; mb < MBW; ++mb) acc[mb] = mfma32<DT_I8>(af[j][kk][mb], bf[j][kk], acc[mb]);
+                for (int mb = 0; mb < MBW; ++mb) acc[mb] = mfma32<DT_I8>(af[jj][kk][mb], bf[jj][kk], acc[mb]);
         __builtin_amdgcn_sched_barrier(0);
     };
     // The groups that still issue copies, then the request for the epilogue's operands (younger than every copy,
@@ -286,10 +308,28 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
     // rest; steps left over by a k slice that is not a multiple of G go one at a time.
     uint32_t s = 0;
     for (; issued < nsteps && s + G <= nsteps; s += G) k_group(s, std::integral_constant<int, G>{});
-    request_epilogue_operands();
+    if (!KP || kp == 0) request_epilogue_operands();
     for (; s + G <= nsteps; s += G) k_group(s, std::integral_constant<int, G>{});
     if constexpr (!AP) {   // (with pairs the host guarantees whole groups)
         for (; s < nsteps; ++s) k_group(s, std::integral_constant<int, 1>{});
+    }
+
+    if constexpr (KP) {   // the two step parities meet: waves 4-7 hand their sums to waves 0-3 and leave
+        CATCOC_WAIT_VMCNT(0);
+        __syncthreads();   // every wave has left the ring
+        int *meet = (int *)smem;   // [4][MBW][16][64]
+        if (kp == 1) {
+#pragma unroll
+            for (int mb = 0; mb < MBW; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) meet[((w * MBW + mb) * 16 + r) * 64 + lane] = acc[mb][r];
+        }
+        __syncthreads();
+        if (kp == 1) return;
+#pragma unroll
+        for (int mb = 0; mb < MBW; ++mb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mb][r] += meet[((w * MBW + mb) * 16 + r) * 64 + lane];
     }
 
     // ---- k slices meet -------------------------------------------------------------
@@ -350,10 +390,10 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         __syncthreads();
         if (*flag != f - 1u) return;
         if (tid == 0) __hip_atomic_store(args.skCount + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // the other slices' partials: every 32-row block of up to three slices per round trip
+        // the other slices' partials: every 32-row block of up to QG slices per round trip
         const int32_t *tile0 = args.skPart + (size_t)tile * (128 * 128);
         const size_t sliceStride = (size_t)loopsM * loopsN * (128 * 128);
-        constexpr int QG = 3;
+        constexpr int QG = (KP && MBW == 4) ? 1 : 3;   // (two waves per SIMD have half the registers each)
         for (uint32_t o0 = 0; o0 + 1 < f; o0 += QG) {
             v4i pv[QG][MBW][4];
             v2i sums[QG];
@@ -441,10 +481,10 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
             }
         float v[16];
         if (redI32) {
-            for (uint32_t p0 = 0; p0 < args.nPeers; p0 += 8) {
+            for (uint32_t p0 = 0; p0 < args.nPeers; p0 += PB) {
                 if (t != mbK || p0 != 0) fetch_peers(k, p0, pv0);
 #pragma unroll
-                for (int q = 0; q < 8; ++q)
+                for (int q = 0; q < PB; ++q)
                     if (p0 + q < args.nPeers) {
 #pragma unroll
                         for (int r = 0; r < 16; ++r) iv[r] += f2i(pv0[q][r]);   // (the loads carry bit patterns)
@@ -458,10 +498,10 @@ __global__ void __launch_bounds__(256, 1) gemm_splitk_kernel(const GemmArgs args
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = __fmul_rn(__fmul_rn((float)iv[r], sN), __shfl(sMt, slot_row(r) + 4 * h, 64));
-        for (uint32_t p0 = 0; p0 < (redI32 ? 0u : args.nPeers); p0 += 8) {
+        for (uint32_t p0 = 0; p0 < (redI32 ? 0u : args.nPeers); p0 += PB) {
             if (t != mbK || p0 != 0) fetch_peers(k, p0, pv0);
 #pragma unroll
-            for (int q = 0; q < 8; ++q)
+            for (int q = 0; q < PB; ++q)
                 if (p0 + q < args.nPeers) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) v[r] = __fadd_rn(v[r], pv0[q][r]);
