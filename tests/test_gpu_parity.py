@@ -1428,6 +1428,72 @@ def test_float_config3_full_size_properties():
         assert abs(csh[task] - want_cs) <= 1e-6 * 128 * 256, task
 
 
+# the shapes the reference's own sweeps run (M, K, N[, Transpose A, Transpose B] rows of its test_shapes.csv files)
+_REFERENCE_SWEEP = [
+    ("allreduce", 16384, 27392, 4096, False, 2, 1, oracle.FP16),       # examples/00_matmul_allreduce/scripts/test_shapes.csv
+    ("allreduce", 131072, 8192, 3072, False, 2, 0, oracle.BF16),
+    ("allgather", 1024, 6148, 5120, False, 8, 3, oracle.FP16),         # examples/01_allgather_matmul/scripts/test_shapes.csv
+    ("reduce_scatter", 16384, 27392, 4096, False, 8, 5, oracle.BF16),  # examples/02_matmul_reduce_scatter/scripts/test_shapes.csv
+    ("reduce_scatter", 131072, 8192, 3072, False, 8, 2, oracle.FP16),
+    ("reduce_scatter", 8192, 27392, 4096, True, 8, 7, oracle.FP16),    # examples/dynamic_tiling/scripts/test_shapes.csv (B as [n,k])
+    ("reduce_scatter", 7936, 12544, 6656, True, 8, 0, oracle.BF16),
+    ("reduce_scatter", 8144, 5120, 1696, True, 8, 4, oracle.FP16),
+]
+
+
+@pytest.mark.parametrize("case", _REFERENCE_SWEEP, ids=lambda c: "%s-%dx%dx%d" % (c[0], c[1], c[2], c[3]))
+def test_float_shapes_of_the_reference_sweeps(case):
+    """Every shape of the reference's test_shapes.csv files at full size (up to 131072 rows, k up to 27392, a k that is
+    not a whole number of 16-byte pieces, row blocks that are not whole tiles, weights as [n,k]): operands of up to
+    2 GiB, so every offset the kernels form is exercised near the top of its range.  A sample of output rows -- the
+    first and the last of the kept block, rows either side of tile boundaries, the rest spread evenly -- against the oracle
+    within the reference's gate and the stated 1e-2."""
+    _need_gpu()
+    op, M, K, N, tb, P, rank, dtype = case
+    tdt = TORCH_DT[dtype]
+    g = torch.Generator(device=DEV).manual_seed(1000 + M % 997)
+
+    def operand(rows, cols, scale):   # generated in slabs: the fp32 draw of a 2 GiB operand would be 4 GiB at once
+        t = torch.empty((rows, cols), dtype=tdt, device=DEV)
+        for r0 in range(0, rows, 8192):
+            r1 = min(rows, r0 + 8192)
+            t[r0:r1] = (torch.randn((r1 - r0, cols), device=DEV, generator=g) * scale).to(tdt)
+        return t
+    Bst = operand(N, K, 0.02) if tb else operand(K, N, 0.02)
+    Bh = host16(Bst)
+    if op == "allgather":
+        shards = [operand(M, K, 1.0) for _ in range(P)]
+        out = ops.allgather_matmul(shards[rank], [shards[r] for r in range(P) if r != rank], Bst, rank, P)
+        torch.cuda.synchronize()
+        rows_all = M * P
+        sel = np.unique(np.concatenate([[0, 127, 128, rows_all - 1, M - 1, M, 3 * M + 5], np.linspace(0, rows_all - 1, 40).astype(np.int64)]))
+        Asel = np.stack([host16(shards[r // M][r % M]) for r in sel])
+        part, want = oracle.matmul_reduce(Asel, Bh, dtype, 0, len(sel), [], want_partial=True)
+        _check_float(host16(out[torch.as_tensor(sel, device=DEV)]), want, part, dtype, K)
+        return
+    A = operand(M, K, 1.0)
+    kept0, kept = (0, M) if op == "allreduce" else (rank * (M // P), M // P)
+    peers = [torch.randn((kept, N), device=DEV, generator=g) for _ in range(P - 1)]
+    if op == "allreduce":
+        out = ops.matmul_allreduce(A, Bst, peers, rank, P, trans_b=tb)
+    else:
+        out = ops.matmul_reduce_scatter(A, Bst, peers, rank, P, trans_b=tb)
+    L.check()
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (kept, N)
+    rel = np.unique(np.concatenate([[0, 1, 127, 128, 255, 256, kept - 129, kept - 128, kept - 2, kept - 1],
+                                    np.linspace(0, kept - 1, 38).astype(np.int64)]))
+    rel = rel[(rel >= 0) & (rel < kept)]
+    idx = torch.as_tensor(rel, device=DEV)
+    Asel = host16(A[idx + kept0])
+    psel = [p[idx].cpu().numpy() for p in peers]
+    part, want = oracle.matmul_reduce(Asel, Bh, dtype, 0, len(rel), psel, transB=tb, want_partial=True)
+    _check_float(host16(out[idx]), want, part + sum(psel), dtype, K)
+    # (sums of up to 27392 products: the blocked fp32 accumulation drifts further from the oracle's k-sequential one than at
+    # the benchmark configs, and elements near zero count many ulps; the gates above are the criterion)
+    _report_ulp("%s %dx%dx%d row sample" % (op, M, K, N), ulp_diff16(host16(out[idx]), want), share=0.99)
+
+
 @pytest.mark.parametrize("case", [(1024, 8192, 8192, 8, 3, None), (512, 8192, 8192, 4, 1, (0, 2)), (1024, 8192, 6144, 2, 0, None)])
 def test_quant_rs_operands_streamed_from_hbm(case):
     """At most one workgroup per CU and 48 MB of operands or more: the launch runs the six-stage ring with the pipelined
