@@ -1494,6 +1494,57 @@ def test_float_shapes_of_the_reference_sweeps(case):
     _report_ulp("%s %dx%dx%d row sample" % (op, M, K, N), ulp_diff16(host16(out[idx]), want), share=0.99)
 
 
+# (M, K, N, weights as [n,k], int32 peers, P, rank or None for explicit kept rows (kept_begin, kept_rows))
+@pytest.mark.parametrize("case", [(16384, 27392, 4096, False, False, 8, 5), (131072, 8192, 3072, False, True, 8, 7),
+                                  (8192, 27392, 4096, True, False, 8, 0), (7936, 12544, 6656, True, False, 8, 3),
+                                  (16, 27392, 16384, True, False, 8, (6, 2)), (128, 27392, 16384, False, True, 8, (96, 32)),
+                                  (512, 16384, 32768, False, False, 8, (448, 64))],
+                         ids=lambda c: "%dx%dx%d" % (c[0], c[1], c[2]))
+def test_quant_shapes_of_the_reference_sweeps(case):
+    """The W8A8 operator at the sizes of the reference's sweeps (its float examples' test_shapes.csv; the quant example's own
+    csv holds the 4x128x512 debug shape, tested elsewhere) and the decode form at the same k with wide n: operands of up
+    to 1 GiB, kept rows anywhere.  A sample of kept rows bit for bit against the oracle."""
+    _need_gpu()
+    M, K, N, tb, ri, P, where = case
+    g = torch.Generator(device=DEV).manual_seed(2000 + M % 997)
+
+    def operand(rows, cols):
+        t = torch.empty((rows, cols), dtype=torch.int8, device=DEV)
+        for r0 in range(0, rows, 16384):
+            r1 = min(rows, r0 + 16384)
+            t[r0:r1] = torch.randint(-127, 128, (r1 - r0, cols), dtype=torch.int8, device=DEV, generator=g)
+        return t
+    x1 = operand(M, K)
+    x2 = operand(N, K) if tb else operand(K, N)
+    s1 = torch.empty(M, device=DEV).uniform_(0.005, 0.02, generator=g)
+    s2 = torch.empty(N, device=DEV).uniform_(0.001, 0.01, generator=g)
+    bias = torch.randint(-1000, 1000, (N,), dtype=torch.int32, device=DEV, generator=g)
+    kb, kr = where if isinstance(where, tuple) else (where * (M // P), M // P)
+    if ri:
+        peers = [torch.randint(-2 ** 24, 2 ** 24, (kr, N), dtype=torch.int32, device=DEV, generator=g) for _ in range(P - 1)]
+    else:
+        peers = [torch.randn((kr, N), device=DEV, generator=g) for _ in range(P - 1)]
+    if isinstance(where, tuple):
+        need, fac, tiles = ops.splitk_plan(M, K, N, P, kb, kr)
+        ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=DEV)
+        out = ops.quant_matmul_splitk(x1, x2, s1, s2, bias, peers, P, kb, kr, workspace=ws, trans_b=tb, reduce_int32=ri)
+    else:
+        out = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, bias, peers, where, P, trans_b=tb, reduce_int32=ri)
+    L.check()
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (kr, N)
+    rel = np.unique(np.concatenate([[0, 1, 31, 32, 127, 128, kr - 129, kr - 128, kr - 2, kr - 1], np.linspace(0, kr - 1, 30).astype(np.int64)]))
+    rel = rel[(rel >= 0) & (rel < kr)]
+    idx = torch.as_tensor(rel, device=DEV)
+    x2h = x2.cpu().numpy()
+    if tb:
+        x2h = np.ascontiguousarray(x2h.T)
+    acc, want = oracle.quant_matmul_reduce_scatter(x1[idx + kb].cpu().numpy(), x2h, s1[idx + kb].cpu().numpy(), s2.cpu().numpy(),
+                                                   bias.cpu().numpy(), 0, len(rel), [p[idx].cpu().numpy() for p in peers], oracle.BF16,
+                                                   reduce_int32=ri)
+    assert np.array_equal(host16(out[idx]), want), "kept rows differ from the oracle"
+
+
 @pytest.mark.parametrize("case", [(1024, 8192, 8192, 8, 3, None), (512, 8192, 8192, 4, 1, (0, 2)), (1024, 8192, 6144, 2, 0, None)])
 def test_quant_rs_operands_streamed_from_hbm(case):
     """At most one workgroup per CU and 48 MB of operands or more: the launch runs the six-stage ring with the pipelined
