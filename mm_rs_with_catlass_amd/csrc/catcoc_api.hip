@@ -123,9 +123,20 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     // tile selection: the fast kernels have n0 = 256 and m0 in {64,128}, or 256 for W8A8 on full tiles
     uint32_t m0 = t->m0, n0 = t->n0;
     if (n0 == 0) n0 = 256;
-    const bool can256 = n0 == 256 && !transA && !transB && mRank % 256 == 0 && t->n % 256 == 0 &&
+    const bool can256 = n0 == 256 && !transA && mRank % 256 == 0 && t->n % 256 == 0 &&
                         ((uint64_t)t->k * es) % 128 == 0;
-    if (m0 == 0) m0 = (mRank <= 64) ? 64 : 128;
+    if (m0 == 0) {
+        // The library's choice: 128-row tiles (two workgroups per CU) unless the launch has at least two 256x256 tiles per CU
+        // and a row of k holds 4 KiB or more: there 256 rows measured 3-10 % faster with B as [k,n] and 15-25 % with B as
+        // [n,k] (8192-row launches, both element types); at 1792 bytes of k (the benchmark shards) 128 rows stay ahead.  The
+        // rule does not look at the layout of B (with [n,k] the larger tile already pays from 2 KiB of k on): the queries for
+        // task counts and workspace sizes do not know the layout and must see the same tiles.  All-gather keeps 128 rows
+        // unless the caller asks.
+        const uint64_t kBytes = (uint64_t)t->k * es;
+        const uint64_t tiles256 = (uint64_t)(t->m / 256u) * (t->n / 256u);
+        const bool pays = tiles256 >= 512 && kBytes >= 4096;
+        m0 = (mRank <= 64) ? 64 : (can256 && pays && op != OP_ALLGATHER) ? 256 : 128;
+    }
     const bool dmaShape = can256 && m0 == 256;
     // (A as [k,m] exists in the 128-row direct-to-LDS kernel only: rows of m in whole 16-byte pieces, a rank's block on that grid)
     const bool taOk = !transA || (m0 == 128 && ((uint64_t)t->m * es) % 16 == 0 && ((uint64_t)mRank * es) % 16 == 0);
@@ -140,7 +151,7 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     const bool ragged = plan.edge && m0 == 128 && mRank >= m0 && t->n >= n0 && ((uint64_t)t->k * es) % 64 == 0 && t->n % 8 == 0 &&
                         (transB || ((uint64_t)t->n * es) % 16 == 0);
     plan.dma = fastShape && (!plan.edge || ragged) && (m0 == 256 || (m0 == 128 && (!transB || ((uint64_t)t->k * es) % 16 == 0))) &&
-               (m0 == 128 || (!transA && !transB));
+               (m0 == 128 || !transA);
     if (transA && !plan.dma) plan.variant = 0;   // the other fast kernels take A as [m,k] only
 
     GemmArgs &a = plan.args;

@@ -12,7 +12,8 @@ int launch_gemm_bf16(const GemmArgs &args, int variant, bool edge, void *stream)
 int launch_gemm_dma_bf16(const GemmArgs &args, void *stream)
 {
     if (args.sched.m0 == 256) {
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
+        if (args.transB) hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4, true>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
+        else hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
         return (int)hipGetLastError();
     }
     return launch_dma_128<DT_BF16>(args, (hipStream_t)stream);

@@ -78,11 +78,12 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 // One LDS pool per workgroup, carved by constant offsets:
 //   128-row tile: three A stages (8 KiB each), then three B stages (16 KiB each)            = 72 KiB
 //   256-row tile: two A pair buffers (32 KiB each), then four B stages (16 KiB each)         = 128 KiB
+//   256-row tile, B as [n][k]: two A pair buffers, then three B pair buffers (32 KiB each)   = 160 KiB, the whole LDS
 // (a 64-row tile of the four-wave geometry uses the first 60 KiB of the 72)
 //   128-row tile, six stages, A in pairs (AQ): four A pair buffers (16 KiB each), then six B stages = 160 KiB, the whole LDS
-template <int WM, int NS = 3, bool AQ = false> struct DmaPool
+template <int WM, int NS = 3, bool AQ = false, bool TB = false> struct DmaPool
 {
-    static constexpr int BYTES = (WM == 4) ? (4 * 256 * 64 + 4 * 64 * 256) : AQ ? ((NS / 2 + 1) * 128 * 128 + NS * 64 * 256) : NS * (128 * 64 + 64 * 256);
+    static constexpr int BYTES = (WM == 4) ? (TB ? 5 * 256 * 128 : 4 * 256 * 64 + 4 * 64 * 256) : AQ ? ((NS / 2 + 1) * 128 * 128 + NS * 64 * 256) : NS * (128 * 64 + 64 * 256);
 };
 
 // One tile (or one k slice of a tile) of the launch: position `pos` of the launch order, in the caller's LDS pool.
@@ -111,7 +112,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     constexpr int A_DMA = BM / 16 / NW;  // 1 KiB copies per wave per stage
     constexpr int B_DMA = 16 / NW;
     constexpr int STEP_DMA = A_DMA + B_DMA;
-    constexpr int POOL = DmaPool<WM, NS, AQ>::BYTES;
+    constexpr int POOL = DmaPool<WM, NS, AQ, TB>::BYTES;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -261,7 +262,14 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     constexpr int B_KK = (ES == 1) ? 32 * 256 : 16 * 512;     // bytes of a stage per 32-byte k slab
     constexpr int B_HALF = (ES == 1) ? 8 * 256 : 4 * 512;     // second transpose read of a fragment
     const uint32_t bt_lds = (wn * 128 + c32) * 64, bt_sw = (c32 >> 2) & 3;   // [n][k] stage: row of column c32, chunk swizzle
+    // 256-row tile with B as [n][k]: B sits in pair buffers like A (rows of 128 bytes, two k steps); bpar = step of the pair
+    uint32_t bpar = 0;
+    const uint32_t bp4_lds = (wn * 128 + c32) * 128, bp4_sw = (c32 >> 1) & 7;
     auto read_b1 = [&](v4i (&bf)[4], const unsigned char *sb, int kk, int nb) {
+        if constexpr (TB && WM == 4) {
+            bf[nb] = *(const v4i *)(sb + bp4_lds + nb * 32 * 128 + (((bpar * 4 + 2 * kk + h) ^ bp4_sw) * 16));
+            return;
+        }
         if constexpr (TB) {
             bf[nb] = *(const v4i *)(sb + bt_lds + nb * 32 * 64 + (((2 * kk + h) ^ bt_sw) * 16));
             return;
@@ -584,6 +592,101 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             wait_steps(nk - 1 - kt);
             barrier_keep_vmem();
             step(false);
+        }
+        mma(fa1, fb1);
+    } else if constexpr (TB) {
+        // ---- 256x256, B as [n][k] ---------------------------------------------------------------------
+        // Both operands are rows of k: both sit in pair buffers (256 rows x 128 bytes = two k steps, whole 128-byte lines per
+        // row), A in two of them, B in three.  Copies are issued at even steps only, after the barrier, in this order:
+        // A pair (kt+2)/2, then B pair (kt+4)/2 -- B runs a pair further ahead.  The barrier of an even step s needs A pair
+        // s/2 (issued in step s-2) and B pair s/2 (in step s-4): younger than both are only the copies of B pair s/2+1.
+        // Odd steps issue nothing, read the buffers their even step waited for and need neither wait nor barrier.
+        // (K in whole pairs of steps: the host requires k * element size to be a multiple of 128.)
+        constexpr int AP = 256 * 128;   // bytes of a pair buffer
+        constexpr int APC = 32 / NW;    // pair copies per wave and operand
+        auto stAP = [&](uint32_t q) { return smem + (q & 1) * AP; };
+        auto stBP = [&](uint32_t q) { return smem + 2 * AP + (q % 3u) * AP; };
+        // pair copy j covers rows 8j..8j+7: lane -> row 8j + lane/8, slot lane&7 holds chunk slot ^ ((row>>1)&7)
+        const unsigned char *gP[APC], *gQ[APC];
+#pragma unroll
+        for (int jj = 0; jj < APC; ++jj) {
+            const int row = 8 * (w + NW * jj) + (lane >> 3);
+            gP[jj] = Ag + (size_t)row * ldaB + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+            gQ[jj] = Bg + (size_t)row * ldbB + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+        }
+        auto issue_ap = [&](uint32_t q) {   // pairs are issued in increasing q
+#pragma unroll
+            for (int jj = 0; jj < APC; ++jj) {
+                dma16_at(gP[jj], lds0 + (q & 1) * AP + (ws + NW * jj) * 1024);
+                gP[jj] += 128;
+            }
+        };
+        auto issue_bp = [&](uint32_t q) {
+#pragma unroll
+            for (int jj = 0; jj < APC; ++jj) {
+                dma16_at(gQ[jj], lds0 + 2 * AP + (q % 3u) * AP + (ws + NW * jj) * 1024);
+                gQ[jj] += 128;
+            }
+        };
+        const uint32_t ap_lds = (wm * 32 * MB + c32) * 128;
+        const uint32_t ap_sw = (c32 >> 1) & 7;
+        auto load_ap = [&](v4i (&af)[MB], uint32_t kt, int kk) {
+            const unsigned char *sa = stAP(kt >> 1) + ap_lds + ((((kt & 1) * 4 + 2 * kk + h) ^ ap_sw) * 16);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) af[mb] = *(const v4i *)(sa + mb * 32 * 128);
+        };
+        auto issue_even_a = [&](uint32_t kt, bool guard) {
+            if ((kt & 1) == 0 && (!guard || kt + 2 < nk)) issue_ap((kt + 2) >> 1);
+        };
+        auto issue_even_b = [&](uint32_t kt, bool guard) {
+            if ((kt & 1) == 0 && (!guard || kt + 4 < nk)) issue_bp((kt + 4) >> 1);
+        };
+        // prologue in steady-state order: A pair 0, B pairs 0 and 1
+        issue_ap(0);
+        issue_bp(0);
+        if (nk > 2) issue_bp(1);
+        // step 0 (peeled: no MFMAs pending yet)
+        if (nk > 2) CATCOC_WAIT_VMCNT(APC);
+        else CATCOC_WAIT_VMCNT(0);
+        barrier_keep_vmem();
+        issue_even_a(0, true);
+        issue_even_b(0, true);
+        bpar = 0;
+        load_ap(fa0, 0, 0);
+        load_b(fb0, stBP(0), 0);
+        load_ap(fa1, 0, 1);
+        load_b(fb1, stBP(0), 1);
+        CATCOC_FENCE();
+        mma(fa0, fb0);
+        CATCOC_FENCE();
+
+        auto compute = [&](uint32_t kt, bool guard) {
+            // The two waves that share a SIMD (w and w + 4) issue their copies in different halves of the step,
+            // so that one of them always has MFMAs to feed the matrix pipe while the other computes addresses.
+            const bool early = ws < NW / 2;
+            bpar = kt & 1u;
+            sched_step([&](v4i (&af)[MB], int kk) { load_ap(af, kt, kk); }, stBP(kt >> 1),
+                       [&] { if (early) issue_even_a(kt, guard); }, [&] { if (early) issue_even_b(kt, guard); }, nothing,
+                       [&] {
+                           if (!early) {
+                               issue_even_a(kt, guard);
+                               issue_even_b(kt, guard);
+                           }
+                       });
+        };
+        uint32_t kt = 1;
+        for (; kt + 6 <= nk; kt += 2) {   // (the even step kt + 1 issues A pair (kt+3)/2 and B pair (kt+5)/2 unguarded)
+            compute(kt, false);
+            CATCOC_WAIT_VMCNT(APC);
+            barrier_keep_vmem();
+            compute(kt + 1, false);
+        }
+        for (; kt < nk; ++kt) {   // tail: drain fully at every even step
+            if ((kt & 1u) == 0) {
+                CATCOC_WAIT_VMCNT(0);
+                barrier_keep_vmem();
+            }
+            compute(kt, true);
         }
         mma(fa1, fb1);
     } else {
@@ -1280,7 +1383,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
 template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false, int NS = 3, bool PP = false, bool AQ = false>
 __global__ void __launch_bounds__(128 * WM, NS == 3 ? 2 : 1) gemm_dma_kernel(const GemmArgs args)
 {
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<WM, NS, AQ>::BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<WM, NS, AQ, TB>::BYTES];
     // A launch with few tiles can cut every tile's k range into kSlices pieces, one workgroup each (128-row tiles
     // only): position `pos` of the launch order runs as kSlices workgroups that stay in the position's XCD column.
     uint32_t pos = blockIdx.x + args.taskBase, slice = 0;   // (taskBase is zero for k-sliced launches)

@@ -13,7 +13,8 @@ int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream)
 int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
 {
     if (args.sched.m0 == 256) {
-        hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
+        if (args.transB) hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, true>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
+        else hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
         return (int)hipGetLastError();
     }
     if (args.flags & GF_ROW_MASK) {   // explicit kept rows in whole 32-row blocks

@@ -304,6 +304,21 @@ def test_quant_rs_m0_256_eight_wave_tile(rank):
     quant_case(np.random.default_rng(33), 2048, 512, 448, 8, rank, tiling=t)
 
 
+# (M, N, K, P, rank): k of one pair of steps, of two, three (an odd number of pairs), four and many; one and several tiles per rank
+@pytest.mark.parametrize("case", [(2048, 512, 128, 8, 0), (2048, 256, 256, 4, 3), (4096, 1024, 384, 8, 6), (2048, 512, 512, 2, 1),
+                                  (4096, 1024, 1920, 8, 5), (2048, 768, 8192, 8, 7)])
+def test_quant_rs_m0_256_weights_stored_n_by_k(case):
+    """The 256x256 tile with B as [n,k]: both operands in pair buffers of whole cache lines (two of A, three of B), copies
+    at even steps only.  Accumulators of every tile bit for bit, kept rows against the oracle, the other ranks' tiles
+    through their checksums; then the int32 reduce order, bias and outbound tiles on the same route."""
+    M, N, K, P, rank = case
+    t = ops.default_tiling(M, K, N, P, m0=256, n0=256, k0=256, commInterval=1)
+    r = quant_case(np.random.default_rng(40 + K), M, N, K, P, rank, tiling=t, trans_b=True, bias=(K % 256 == 0))
+    assert r["exact"] == r["total"]
+    if K == 1920:
+        quant_case(np.random.default_rng(41), M, N, K, P, rank, tiling=t, trans_b=True, reduce_int32=True, outbound=True, stages=4)
+
+
 @pytest.mark.parametrize("case", [(8192, 1024, 512, 8, 0), (8192, 1024, 512, 8, 5), (4096, 2048, 128, 4, 3),
                                   (4096, 2048, 1792, 8, 7), (8192, 1024, 3584, 2, 1)])
 def test_quant_rs_many_tiles_two_launches(case):
@@ -877,6 +892,29 @@ def test_float_reduce_scatter_256_row_tiles_outbound_and_checksum(dtype):
                 assert np.abs(ob - blk).max() <= 1e-2 * max(1.0, np.abs(blk).max()), task
 
 
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+@pytest.mark.parametrize("shape", [(4096, 512, 320, 8, 6), (2048, 1024, 4096, 4, 0), (1024, 256, 64, 2, 1)])
+def test_float_reduce_scatter_256_row_tiles_weights_stored_n_by_k(dtype, shape):
+    # 256x256 tiles with B as [n,k] (the layout of the reference's dynamic_tiling sweep shapes): pair buffers for both operands
+    _need_gpu()
+    M, N, K, P, rank = shape
+    rng = np.random.default_rng(23 + K)
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    part, want = oracle.matmul_reduce(A, B, dtype, rank * rows, rows, peers, want_partial=True)
+    t = ops.default_tiling(M, K, N, P, m0=256, n0=256, k0=256)
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    out = ops.matmul_reduce_scatter(dev16(A, dtype), dev16(np.ascontiguousarray(B.T), dtype), [dev(p) for p in peers], rank, P, tiling=t,
+                                    trans_b=True, acc_dump=dump)
+    L.check()
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part[rank * rows:(rank + 1) * rows] + sum(peers), dtype, K)
+    _report_ulp("256-row tiles, B as [n,k]", ulp_diff16(host16(out), want))
+    assert np.abs(dump.cpu().numpy() - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
+
+
 def test_float_allreduce_config1_full_size():
     # BASELINE config 1: A[512,2048], B[2048,1024] fp16 ~U(-1,1), K halves as the two ranks' partials
     _need_gpu()
@@ -1169,6 +1207,44 @@ def test_pipelined_quant_equals_fused_int32_reduce_and_oracle(case):
         assert np.array_equal(obh[ws.value:ws.value + rv, :cv], acc_want[r0:r0 + rv, c0:c0 + cv]), task
         checked += 1
     assert checked > 0
+
+
+@pytest.mark.parametrize("tb", [False, True])
+def test_pipelined_quant_on_the_librarys_256_row_tiles(tb):
+    """A shape large enough for the library to choose 256x256 tiles by itself (8192x4096x8192, tiling m0 = 0), in both weight
+    layouts: the round-pipelined operator (GEMM rounds of 256-row tiles, comm rounds, int32 reduce) against the fused
+    int32-reduce launch bit for bit, and a sample of kept rows against the oracle."""
+    _need_gpu()
+    import ctypes as C
+    M, N, K, P, rank = 8192, 8192, 4096, 8, 6
+    g = torch.Generator(device=DEV).manual_seed(77)
+    x1 = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=DEV, generator=g)
+    x2 = torch.randint(-127, 128, (N, K) if tb else (K, N), dtype=torch.int8, device=DEV, generator=g)
+    s1 = torch.empty(M, device=DEV).uniform_(0.005, 0.02, generator=g)
+    s2 = torch.empty(N, device=DEV).uniform_(0.001, 0.01, generator=g)
+    rows = M // P
+    peers = [torch.randint(-2 ** 24, 2 ** 24, (rows, N), dtype=torch.int32, device=DEV, generator=g) for _ in range(P - 1)]
+    t = ops.default_tiling(M, K, N, P, m0=0, n0=0, k0=0, commInterval=1)
+    d = L.make_desc(rank, P, [16] * (P - 1))
+    ntasks = L.load().catcoc_get_task_count(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d))
+    assert ntasks == 1024          # 32 x 32 tiles of 256 x 256
+    ob = _outbound_for(L.QUANT_MATMUL_REDUCE_SCATTER, L.INT8, t, rank, P, torch.int32)
+    side = torch.cuda.Stream()
+    out, cacc = ops.pipelined_quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, rank, P, ob, tiling=t, comm_stream=side, trans_b=tb)
+    L.check()
+    torch.cuda.synchronize()
+    fused = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, peers, rank, P, tiling=t, trans_b=tb, reduce_int32=True)
+    torch.cuda.synchronize()
+    assert torch.equal(fused.view(torch.int16), out.view(torch.int16))
+    sel = np.array([0, 1, 255, 256, 511, 700, rows - 1])
+    idx = torch.as_tensor(sel, device=DEV)
+    x2h = x2.cpu().numpy()
+    if tb:
+        x2h = np.ascontiguousarray(x2h.T)
+    acc, want = oracle.quant_matmul_reduce_scatter(x1[idx + rank * rows].cpu().numpy(), x2h, s1[idx + rank * rows].cpu().numpy(), s2.cpu().numpy(),
+                                                   None, 0, len(sel), [p[idx].cpu().numpy() for p in peers], oracle.BF16, reduce_int32=True)
+    assert np.array_equal(host16(out[idx]), want)
+    assert np.array_equal(cacc[idx].cpu().numpy(), acc + sum(p[idx].cpu().numpy() for p in peers))
 
 
 @pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
