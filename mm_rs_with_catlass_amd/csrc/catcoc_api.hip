@@ -127,14 +127,15 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
                         ((uint64_t)t->k * es) % 128 == 0;
     if (m0 == 0) {
         // The library's choice: 128-row tiles (two workgroups per CU) unless the launch has at least two 256x256 tiles per CU
-        // and a row of k holds 4 KiB or more: there 256 rows measured 3-10 % faster with B as [k,n] and 15-25 % with B as
-        // [n,k] (8192-row launches, both element types); at 1792 bytes of k (the benchmark shards) 128 rows stay ahead.  The
+        // and a row of k holds 4 KiB or more (or four per CU and 2 KiB): there 256 rows measured 3-10 % faster with B as
+        // [k,n] and 15-25 % with B as [n,k] (8192-row launches, both element types, launches alternating); with two tiles
+        // per CU and 1792 bytes of k (the benchmark shards) 128 rows stay ahead, 68.8 against 75.7 us.  The
         // rule does not look at the layout of B (with [n,k] the larger tile already pays from 2 KiB of k on): the queries for
         // task counts and workspace sizes do not know the layout and must see the same tiles.  All-gather keeps 128 rows
         // unless the caller asks.
         const uint64_t kBytes = (uint64_t)t->k * es;
         const uint64_t tiles256 = (uint64_t)(t->m / 256u) * (t->n / 256u);
-        const bool pays = tiles256 >= 512 && kBytes >= 4096;
+        const bool pays = (tiles256 >= 512 && kBytes >= 4096) || (tiles256 >= 1024 && kBytes >= 2048);
         m0 = (mRank <= 64) ? 64 : (can256 && pays && op != OP_ALLGATHER) ? 256 : 128;
     }
     const bool dmaShape = can256 && m0 == 256;
