@@ -123,8 +123,11 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     // tile selection: the fast kernels have n0 = 256 and m0 in {64,128}, or 256 for W8A8 on full tiles
     uint32_t m0 = t->m0, n0 = t->n0;
     if (n0 == 0) n0 = 256;
-    const bool can256 = n0 == 256 && !transA && mRank % 256 == 0 && t->n % 256 == 0 &&
-                        ((uint64_t)t->k * es) % 128 == 0;
+    // 256-row tiles: k in whole pairs of 64-byte steps; full tiles, or ragged rows / columns with a whole tile to move an edge
+    // tile into and the moved tile's first column on the 16-byte grid of B, D and the peers (as for 128-row tiles below)
+    const bool full256 = mRank % 256 == 0 && t->n % 256 == 0;
+    const bool can256 = n0 == 256 && !transA && ((uint64_t)t->k * es) % 128 == 0 &&
+                        (full256 || (mRank >= 256 && t->n >= 256 && t->n % 8 == 0 && (transB || ((uint64_t)t->n * es) % 16 == 0)));
     if (m0 == 0) {
         // The library's choice: 128-row tiles (two workgroups per CU) unless the launch has at least two 256x256 tiles per CU
         // and a row of k holds 4 KiB or more (or four per CU and 2 KiB): there 256 rows measured 3-10 % faster with B as
@@ -149,8 +152,9 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
     // (B as [n,k] runs the 128-row direct-to-LDS kernel when its rows of k are 16-byte multiples)
     // Ragged rows / columns on 128-row tiles: the direct-to-LDS kernel moves the edge tiles inwards (GF_RAGGED).  It needs a whole
     // tile to move into, k in whole 64-byte steps, and the moved tile's first column on the 16-byte grid of B, D and the peers.
-    const bool ragged = plan.edge && m0 == 128 && mRank >= m0 && t->n >= n0 && ((uint64_t)t->k * es) % 64 == 0 && t->n % 8 == 0 &&
-                        (transB || ((uint64_t)t->n * es) % 16 == 0);
+    const bool ragged = plan.edge && ((m0 == 128 && mRank >= m0 && t->n >= n0 && ((uint64_t)t->k * es) % 64 == 0 && t->n % 8 == 0 &&
+                                       (transB || ((uint64_t)t->n * es) % 16 == 0)) ||
+                                      (m0 == 256 && can256));
     plan.dma = fastShape && (!plan.edge || ragged) && (m0 == 256 || (m0 == 128 && (!transB || ((uint64_t)t->k * es) % 16 == 0))) &&
                (m0 == 128 || !transA);
     if (transA && !plan.dma) plan.variant = 0;   // the other fast kernels take A as [m,k] only

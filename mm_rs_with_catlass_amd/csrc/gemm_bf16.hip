@@ -12,8 +12,12 @@ int launch_gemm_bf16(const GemmArgs &args, int variant, bool edge, void *stream)
 int launch_gemm_dma_bf16(const GemmArgs &args, void *stream)
 {
     if (args.sched.m0 == 256) {
-        if (args.transB) hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4, true>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
-        else hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
+        const dim3 grid(launch_positions(args)), block(512);
+        const bool ragged = (args.flags & GF_RAGGED) != 0;   // edge tiles moved inwards, as on 128-row tiles
+        if (args.transB && ragged) hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4, true, false, true>), grid, block, 0, (hipStream_t)stream, args);
+        else if (args.transB) hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4, true>), grid, block, 0, (hipStream_t)stream, args);
+        else if (ragged) hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4, false, false, true>), grid, block, 0, (hipStream_t)stream, args);
+        else hipLaunchKernelGGL((gemm_dma_kernel<DT_BF16, 4>), grid, block, 0, (hipStream_t)stream, args);
         return (int)hipGetLastError();
     }
     return launch_dma_128<DT_BF16>(args, (hipStream_t)stream);

@@ -97,7 +97,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                                          uint32_t subRow)
 {
     static_assert(!RM || (DT == DT_I8 && WM == 2), "row-mask mode exists for the W8A8 128-row kernel");
-    static_assert(!RG || (WM == 2 && !RM), "ragged mode exists for the 128-row kernel");
+    static_assert(!RG || !RM, "ragged mode and row-mask mode exclude each other");
     static_assert(!TA || (WM == 2 && !RM), "transposed A exists for the 128-row kernel");
     static_assert(WM == 2 || WM == 4, "supported geometries");
     static_assert(NS == 3 || (WM == 2 && NS >= 3 && NS <= 8), "deeper rings exist for the 128-row kernel");

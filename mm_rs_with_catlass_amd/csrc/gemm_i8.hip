@@ -13,8 +13,12 @@ int launch_gemm_i8(const GemmArgs &args, int variant, bool edge, void *stream)
 int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
 {
     if (args.sched.m0 == 256) {
-        if (args.transB) hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, true>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
-        else hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), dim3(launch_positions(args)), dim3(512), 0, (hipStream_t)stream, args);
+        const dim3 grid(launch_positions(args)), block(512);
+        const bool ragged = (args.flags & GF_RAGGED) != 0;   // edge tiles moved inwards, as on 128-row tiles
+        if (args.transB && ragged) hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, true, false, true>), grid, block, 0, (hipStream_t)stream, args);
+        else if (args.transB) hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, true>), grid, block, 0, (hipStream_t)stream, args);
+        else if (ragged) hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4, false, false, true>), grid, block, 0, (hipStream_t)stream, args);
+        else hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 4>), grid, block, 0, (hipStream_t)stream, args);
         return (int)hipGetLastError();
     }
     if (args.flags & GF_ROW_MASK) {   // explicit kept rows in whole 32-row blocks

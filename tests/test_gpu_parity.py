@@ -195,6 +195,74 @@ def test_quant_rs_ragged_problem_on_many_tiles(case):
     assert seen_ragged > 0 and seen_full >= 64 and r["ntasks"] <= 256
 
 
+# (M, N, K, P, rank, weights as [n,k], outbound tiles instead of checksums)
+@pytest.mark.parametrize("case", [(8 * 296, 1344, 512, 8, 6, False, False), (8 * 296, 1280, 256, 8, 0, True, True),
+                                  (4 * 1064, 1088, 128, 4, 3, True, False), (2 * 1000, 2120, 384, 2, 1, False, True),
+                                  (8 * 300, 520, 1024, 8, 7, True, False)])
+def test_quant_rs_ragged_problem_on_256_row_tiles(case):
+    """Ragged rows and / or columns on 256x256 tiles (m0 = 256): edge tiles are computed as whole tiles moved up / left until
+    they end at the edge, on the direct-to-LDS kernel in both layouts of B.  Accumulators of every element, the kept
+    block, and every other tile's own part through its checksum or its outbound tile."""
+    import ctypes as C
+    M, N, K, P, rank, tb, outbound = case
+    t = ops.default_tiling(M, K, N, P, m0=256, n0=256, k0=256, commInterval=1)
+    r = quant_case(np.random.default_rng(95 + rank), M, N, K, P, rank, bias=True, tiling=t, trans_b=tb, outbound=outbound, stages=4)
+    d = L.make_desc(rank, P, [16] * (P - 1), stages=4)
+    so = L.load()
+    tr, row, col, ws = (C.c_uint32() for _ in range(4))
+    rows = M // P
+    seen_ragged = 0
+    deq = oracle.dequant(r["acc"], r["s2"], r["s1"]) if outbound else None
+    ob = r["outbound"].cpu().numpy().reshape(-1, 256) if outbound else None
+    cs = r["checksum"].cpu().numpy()
+    for task in range(r["ntasks"]):
+        so.catcoc_task_tile(L.QUANT_MATMUL_REDUCE_SCATTER, C.byref(t), C.byref(d), task, C.byref(tr), C.byref(row), C.byref(col), C.byref(ws))
+        rv = min(256, (tr.value + 1) * rows - row.value)
+        cv = min(256, N - col.value)
+        seen_ragged += rv < 256 or cv < 256
+        if tr.value == rank:
+            continue
+        blk = r["acc"][row.value:row.value + rv, col.value:col.value + cv]
+        if outbound:
+            want = deq[row.value:row.value + rv, col.value:col.value + cv]
+            assert np.array_equal(ob[ws.value:ws.value + rv, :cv].view(np.uint32), want.view(np.uint32)), task
+        else:
+            assert cs[task] == int(blk.astype(np.int64).sum()), task
+    assert seen_ragged > 0
+
+
+@pytest.mark.parametrize("dtype", [oracle.FP16, oracle.BF16])
+@pytest.mark.parametrize("tb", [False, True])
+def test_float_ragged_problems_on_256_row_tiles(dtype, tb):
+    # reduce-scatter with ragged rows and columns and all-reduce with ragged rows on 256x256 tiles, both layouts of B
+    _need_gpu()
+    rng = np.random.default_rng(27)
+    M, N, K, P, rank = 8 * 296, 1344, 448, 8, 5
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    rows = M // P
+    peers = [rng.standard_normal((rows, N)).astype(np.float32) for _ in range(P - 1)]
+    part, want = oracle.matmul_reduce(A, B, dtype, rank * rows, rows, peers, want_partial=True)
+    dump = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    t = ops.default_tiling(M, K, N, P, m0=256, n0=256, k0=256)
+    Bd = dev16(np.ascontiguousarray(B.T) if tb else B, dtype)
+    out = ops.matmul_reduce_scatter(dev16(A, dtype), Bd, [dev(p) for p in peers], rank, P, tiling=t, trans_b=tb, acc_dump=dump)
+    L.check()
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part[rank * rows:(rank + 1) * rows] + sum(peers), dtype, K)
+    assert np.abs(dump.cpu().numpy() - part).max() <= 1e-2 * max(1.0, np.abs(part).max())
+    M, N, K = 1100, 2048, 320
+    A = _rand16(rng, (M, K), dtype)
+    B = _rand16(rng, (K, N), dtype, 0.02)
+    p1 = rng.standard_normal((M, N)).astype(np.float32)
+    part, want = oracle.matmul_reduce(A, B, dtype, 0, M, [p1], want_partial=True)
+    t = ops.default_tiling(M, K, N, 2, m0=256, n0=256, k0=256)
+    out = ops.matmul_allreduce(dev16(A, dtype), dev16(np.ascontiguousarray(B.T) if tb else B, dtype), [dev(p1)], 0, 2, tiling=t, trans_b=tb)
+    L.check()
+    torch.cuda.synchronize()
+    _check_float(host16(out), want, part + p1, dtype, K)
+
+
 @pytest.mark.parametrize("tb", [False, True])
 def test_quant_rs_kept_tiles_whole_or_split_give_the_same_bits(tb):
     # CATCOC_FLAG_KEPT_WHOLE / CATCOC_FLAG_KEPT_SPLIT are tuning knobs: output, kept accumulators and checksums must not change
