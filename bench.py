@@ -235,6 +235,23 @@ def float_configs(args, torch, L, ops, dev):
     wall, kern = timed(lambda: ops.matmul_allreduce(A1, B1, peer, 0, P, out=out1, workspace=ws1))
     res.append({"config": 1, "op": "matmul_allreduce fp16 M=512 K=1024(local) N=1024 P=2", "kernel_us": round(kern * 1e6, 2),
                 "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * M * N * K / kern / 1e12, 1), "k_slices": f1})
+    # the two large shapes of the reference's own sweep (examples/dynamic_tiling/scripts/test_shapes.csv: fp16, B stored as
+    # [n,k]), tile left to the library (256 rows here; the second shape has 992 rows per rank: ragged tiles)
+    del A, B, peers, shards, B2
+    for M, K, N in ((8192, 27392, 4096), (7936, 12544, 6656)):
+        P, rank = 8, 0
+        A = torch.randn((M, K), device=dev, generator=g).half()
+        B = (torch.randn((N, K), device=dev, generator=g) * 0.02).half()
+        peers = [torch.randn((M // P, N), device=dev, generator=g) for _ in range(P - 1)]
+        outs = torch.empty((M // P, N), dtype=torch.float16, device=dev)
+        wall, kern = timed(lambda: ops.matmul_reduce_scatter(A, B, peers, rank, P, trans_b=True, out=outs))
+        t128 = ops.default_tiling(M, K, N, P, m0=128, n0=256, k0=256)
+        _, kern128 = timed(lambda: ops.matmul_reduce_scatter(A, B, peers, rank, P, trans_b=True, out=outs, tiling=t128))
+        tf = 2.0 * M * N * K / kern / 1e12
+        res.append({"config": "reference sweep shape", "op": "matmul_reduce_scatter fp16 M=%d K=%d N=%d P=8, B as [n,k]" % (M, K, N),
+                    "kernel_us": round(kern * 1e6, 1), "wall_us": round(wall * 1e6, 1), "TFLOPS": round(tf, 1),
+                    "mfma_frac": round(tf / PEAK_F16_TFLOPS, 4), "kernel_us_on_128_row_tiles": round(kern128 * 1e6, 1)})
+        del A, B, peers
     c3 = res[0]
     print(json.dumps({
         "metric": "fp16 matmul-reduce-scatter shard (BASELINE config 3) TFLOPS, 1 MI355X", "value": c3["TFLOPS"], "unit": "TFLOPS",
