@@ -30,7 +30,8 @@ PERF_TEST_CYCLE_TIMES = 3   # info.h:23
 
 def candidates(rows_per_rank, full_tiles):
     """The MI355X-side search space for one shape: (m0, (swizzle offset, direction), linear order, commInterval)."""
-    m0s = [128] + ([256] if full_tiles and rows_per_rank % 256 == 0 else []) + ([64] if rows_per_rank <= 64 else [])
+    # (256-row tiles take ragged problems too, from one whole tile of rows per rank on; the library rejects what it cannot run)
+    m0s = [128] + ([256] if rows_per_rank >= 256 else []) + ([64] if rows_per_rank <= 64 else [])
     out = []
     for m0 in m0s:
         for swz in ((7, 1), (3, 0)):

@@ -521,7 +521,8 @@ def test_sweep_csv_has_the_reference_columns_and_best_pick(tmp_path):
     best = tuning.best_results(rows)
     assert len(best) == 2 and {b["Time(us)"] for b in best} == {71.5, 5.0}
     assert (tuning.WARM_UP_TIMES, tuning.PERF_TEST_CYCLE_TIMES) == (10, 3)      # examples/dynamic_tiling/include/info.h:22-23
-    assert (256, (7, 1), False, 1) in tuning.candidates(1024, True) and all(c[0] != 256 for c in tuning.candidates(1018, False))
+    assert (256, (7, 1), False, 1) in tuning.candidates(1024, True) and (256, (3, 0), True, 4) in tuning.candidates(1018, False)
+    assert all(c[0] != 256 for c in tuning.candidates(200, False)) and (64, (7, 1), False, 1) in tuning.candidates(64, True)
 
 
 def test_task_tiles_batch_query_equals_single_queries(so):
