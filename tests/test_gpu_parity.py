@@ -1013,6 +1013,14 @@ def test_allgather_matmul_reads_shards_in_place(dtype, shape):
     torch.cuda.synchronize()
     full = oracle.gemm_half_f32(np.concatenate(shards, 0), B, dtype)
     _check_float(host16(out), want, full, dtype, K)
+    if ml % 256 == 0 and N % 256 == 0:     # the same on 256x256 tiles, in both layouts of B
+        t = ops.default_tiling(ml, K, N, P, m0=256, n0=256, k0=256)
+        for tb in (False, True):
+            Bd = dev16(np.ascontiguousarray(B.T) if tb else B, dtype)
+            out = ops.allgather_matmul(dsh[rank], [dsh[r] for r in range(P) if r != rank], Bd, rank, P, tiling=t, trans_b=tb)
+            L.check()
+            torch.cuda.synchronize()
+            _check_float(host16(out), want, full, dtype, K)
 
 
 @pytest.mark.parametrize("kslices", [False, True])
