@@ -236,7 +236,8 @@ def float_configs(args, torch, L, ops, dev):
     res.append({"config": 1, "op": "matmul_allreduce fp16 M=512 K=1024(local) N=1024 P=2", "kernel_us": round(kern * 1e6, 2),
                 "wall_us": round(wall * 1e6, 2), "TFLOPS": round(2.0 * M * N * K / kern / 1e12, 1), "k_slices": f1})
     # the two large shapes of the reference's own sweep (examples/dynamic_tiling/scripts/test_shapes.csv: fp16, B stored as
-    # [n,k]), tile left to the library (256 rows here; the second shape has 992 rows per rank: ragged tiles)
+    # [n,k]) on 256-row tiles (the library's own choice for the first; the second has 992 rows per rank, ragged tiles, which
+    # take 256 rows on request)
     del A, B, peers, shards, B2
     for M, K, N in ((8192, 27392, 4096), (7936, 12544, 6656)):
         P, rank = 8, 0
@@ -244,7 +245,8 @@ def float_configs(args, torch, L, ops, dev):
         B = (torch.randn((N, K), device=dev, generator=g) * 0.02).half()
         peers = [torch.randn((M // P, N), device=dev, generator=g) for _ in range(P - 1)]
         outs = torch.empty((M // P, N), dtype=torch.float16, device=dev)
-        wall, kern = timed(lambda: ops.matmul_reduce_scatter(A, B, peers, rank, P, trans_b=True, out=outs))
+        t256 = ops.default_tiling(M, K, N, P, m0=256 if (M // P) % 256 else 0, n0=256 if (M // P) % 256 else 0, k0=0)
+        wall, kern = timed(lambda: ops.matmul_reduce_scatter(A, B, peers, rank, P, trans_b=True, out=outs, tiling=t256))
         t128 = ops.default_tiling(M, K, N, P, m0=128, n0=256, k0=256)
         _, kern128 = timed(lambda: ops.matmul_reduce_scatter(A, B, peers, rank, P, trans_b=True, out=outs, tiling=t128))
         tf = 2.0 * M * N * K / kern / 1e12

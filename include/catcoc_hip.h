@@ -27,7 +27,7 @@ extern "C" {
 /* examples/dynamic_tiling/include/info.h:29-42 -- twelve uint32_t, same order.
  * m,k,n: problem (for ALLGATHER_MATMUL m is the rows of ONE rank's shard).
  * m0,n0,k0: workgroup macro tile; 0 lets the library choose (m0: 64 for at most 64 rows per rank, else 128, or 256 when
- * the launch has 512 or more full 256x256 tiles and 4 KiB or more of k per row, or 1024 and 2 KiB; the choice does not depend on the
+ * the problem is whole 256x256 tiles, 512 or more of them with 4 KiB or more of k per row, or 1024 with 2 KiB; the choice does not depend on the
  * operands' layouts, so catcoc_get_task_count / catcoc_get_workspace_size see the same tiles as the launch).
  * commInterval x blockNum: tiles per scheduling round (blockNum, the
  * reference's BLOCK_NUM = 20 AI cores, comes from CatcocSymmetricDesc).

@@ -139,7 +139,8 @@ int make_plan(int commType, int dataType, const CocTilingParams *t, const Catcoc
         const uint64_t kBytes = (uint64_t)t->k * es;
         const uint64_t tiles256 = (uint64_t)(t->m / 256u) * (t->n / 256u);
         const bool pays = (tiles256 >= 512 && kBytes >= 4096) || (tiles256 >= 1024 && kBytes >= 2048);
-        m0 = (mRank <= 64) ? 64 : (can256 && pays && op != OP_ALLGATHER) ? 256 : 128;
+        // (full tiles only: ragged problems take 256 rows on request, since the pipelined operators run those on other kernels)
+        m0 = (mRank <= 64) ? 64 : (can256 && full256 && pays && op != OP_ALLGATHER) ? 256 : 128;
     }
     const bool dmaShape = can256 && m0 == 256;
     // (A as [k,m] exists in the 128-row direct-to-LDS kernel only: rows of m in whole 16-byte pieces, a rank's block on that grid)
