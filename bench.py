@@ -453,6 +453,22 @@ def main():
     torch.cuda.synchronize()
     kern_ms = [a.elapsed_time(b) for a, b in evs]
 
+    # the same launches with all-zero int8 operands (scales, peers and shapes unchanged): identical instruction stream and
+    # memory traffic, far fewer toggling bits in the LDS, register-file and MFMA data paths.  The gap to the timed figure is
+    # what the board's power limit takes at the workload's random operands (the clock drops); this leg only shows it
+    zero_kernel_s = None
+    if not args.no_other_mode:
+        zsets = []
+        for st in sets[:2]:
+            zsets.append(dict(st, x1=torch.zeros_like(st["x1"]), x2=torch.zeros_like(st["x2"]), out=torch.empty_like(st["out"])))
+        zsteps = []
+        for st in zsets:
+            kw = {"outbound": outbound} if args.mode == "outbound" else {"checksum": torch.zeros(ntasks, dtype=torch.int64, device=dev)}
+            zsteps.append(ops.prepare_quant_matmul_reduce_scatter(st["x1"], st["x2"], st["s1"], st["s2"], None, st["peers"], rank, P,
+                                                                  tiling=tiling, out=st["out"], **kw)[0])
+        run(zsteps, max(args.warmup, 10))
+        _, zero_kernel_s = run(zsteps, args.steps)
+
     # the other store mode, as a secondary object: the reference stores the 7/8 non-kept tiles for its peers to pull
     other_mode = "kept" if args.mode == "outbound" else "outbound"
     other = None
@@ -552,6 +568,9 @@ def main():
                      "sustained_note": "%d more launches in ten event-bracketed groups after the timed steps; "
                                        "kernel_us_sustained = mean of the last five groups" % (grp * 10) if series else None,
                      "single_launch_us_min": round(min(kern_ms) * 1e3, 2),
+                     "kernel_us_zero_operands": round(zero_kernel_s * 1e6, 2) if zero_kernel_s else None,
+                     "zero_operands_note": "same launches with all-zero int8 operands (two input sets rotating): same instructions "
+                                           "and traffic, less switching power; not a result, the gap to kernel_us_avg is the power limit" if zero_kernel_s else None,
                      "algorithmic_bytes": int(alg_bytes),
                      "hbm_frac_at_algorithmic_bytes": round(alg_bytes / avg_kernel_s / 1e9 / PEAK_HBM_GBS, 4)},
         "device": info,
