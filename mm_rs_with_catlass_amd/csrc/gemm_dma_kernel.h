@@ -62,6 +62,9 @@ __device__ __forceinline__ void dma16_stream(const unsigned char *g, unsigned ch
 // Geometries (every wave computes 64 x 128: MB = 2 row blocks of 32, 4 column blocks of 32; two wave columns):
 //   WM 2 -> 128x256 tile, 4 waves, 3 stages (72 KiB LDS, two workgroups per CU);
 //   WM 4 -> 256x256 tile, 8 waves (128 KiB LDS, one workgroup per CU): half the L2 -> LDS traffic per MAC.
+//   W8   -> the 128x256 tile on EIGHT waves (four wave rows of 32 rows, MB = 1; WM stays 2: every tile-level rule of the
+//           128-row geometry applies): for the six-stage ring, whose launches have one workgroup per CU -- with four waves
+//           every wave is alone on its SIMD and pays barrier, LDS latency and copy issue of every k step one after the other.
 //   TB   -> B is given as [n][k] (k contiguous, the layout of a weight matrix stored output-major): its tiles are then
 //           staged and read exactly like A's, rows of 64 bytes of k, and need no transposing LDS reads.
 //   RM   -> explicit kept rows (GF_ROW_MASK): the kept rows are whole 32-row blocks anywhere in the row range, so a tile can
@@ -87,12 +90,12 @@ template <int WM, int NS = 3, bool AQ = false, bool TB = false> struct DmaPool
 };
 
 // One tile (or one k slice of a tile) of the launch: position `pos` of the launch order, in the caller's LDS pool.
-// MB = 32-row blocks per wave (2; 1 = a 64-row tile, four-wave geometry only); subRow = first row of a 64-row tile inside
-// its 128-row tile of the schedule.
+// MB = 32-row blocks per wave (2; 1 = a 64-row tile of the four-wave geometry, or the eight-wave geometry W8); subRow =
+// first row of a 64-row tile inside its 128-row tile of the schedule.
 // AQ = A is copied per pair of k steps, 128 bytes per row (whole cache lines: half as many requests to L2 as two 64-byte
 // halves), as the 256-row geometry does; for the six-stage ring, whose launches have one workgroup per CU and feel every
 // request (with three stages and two workgroups per CU the same change measured slower).
-template <uint32_t DT, int WM, bool TB, bool RM, bool RG, bool TA, int MB, int NS = 3, bool PP = false, bool AQ = false>
+template <uint32_t DT, int WM, bool TB, bool RM, bool RG, bool TA, int MB, int NS = 3, bool PP = false, bool AQ = false, bool W8 = false>
 __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *smem, uint32_t pos, uint32_t slice, uint32_t kSlices,
                                          uint32_t subRow)
 {
@@ -101,12 +104,16 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
     static_assert(!TA || (WM == 2 && !RM), "transposed A exists for the 128-row kernel");
     static_assert(WM == 2 || WM == 4, "supported geometries");
     static_assert(NS == 3 || (WM == 2 && NS >= 3 && NS <= 8), "deeper rings exist for the 128-row kernel");
-    static_assert(MB == 2 || (MB == 1 && WM == 2 && !RM && !RG && !TA), "64-row tiles exist for the four-wave geometry with A as [m,k]");
-    static_assert(!AQ || (WM == 2 && NS == 6 && MB == 2 && !TA), "pairs of A steps exist for the six-stage 128-row kernel with A as [m,k]");
+    static_assert(MB == 2 || (MB == 1 && WM == 2 && (!RM || W8) && !RG && !TA), "64-row tiles exist for the four-wave geometry with A as [m,k]");
+    static_assert(!W8 || (WM == 2 && MB == 1 && !RG && !TA), "eight waves on the 128-row tile: 32 rows per wave");
+    static_assert(!AQ || (WM == 2 && NS == 6 && (MB == 2 || W8) && !TA), "pairs of A steps exist for the six-stage 128-row kernel with A as [m,k]");
     using Acc = typename AccOf<DT>::type;
     constexpr int ES = (DT == DT_I8) ? 1 : 2;   // bytes per operand element; a k step is 64 BYTES of K
-    constexpr int NW = 2 * WM;          // waves
-    constexpr int BM = 32 * MB * WM;
+    constexpr int WR = W8 ? 4 : WM;     // wave rows (two wave columns)
+    constexpr int NW = 2 * WR;          // waves
+    constexpr int NT = 64 * NW;         // threads
+    constexpr int BM = 32 * MB * WR;
+    constexpr bool HALF = MB == 1 && !W8;   // a 64-row half of a 128-row tile of the schedule
     constexpr int A_STAGE = BM * 64;
     constexpr int B_STAGE = 64 * 256;
     constexpr int A_DMA = BM / 16 / NW;  // 1 KiB copies per wave per stage
@@ -141,7 +148,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
         task_tile(sp, task, tg);
         ti = tg;
     }
-    if constexpr (MB == 1) {
+    if constexpr (HALF) {
         ti.row += subRow;
         ti.rowInRank += subRow;
         ti.wsRow += subRow;
@@ -823,7 +830,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                         for (int g = 0; g < 4; ++g) {
                             const auto e0 = acc[mb][nb][4 * g], e1 = acc[mb][nb][4 * g + 1], e2 = acc[mb][nb][4 * g + 2], e3 = acc[mb][nb][4 * g + 3];
                             const v4i iv = {__builtin_bit_cast(int, e0), __builtin_bit_cast(int, e1), __builtin_bit_cast(int, e2), __builtin_bit_cast(int, e3)};
-                            __builtin_amdgcn_raw_buffer_store_b128(iv, mine, (((mb * 4 + nb) * 4 + g) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+                            __builtin_amdgcn_raw_buffer_store_b128(iv, mine, (((mb * 4 + nb) * 4 + g) * NT + tid) * 16, 0, DEVICE_SCOPE);
                         }
                 } else if constexpr (RM) {
                     if (args.checksum != nullptr) {
@@ -833,7 +840,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
 #pragma unroll
                             for (int r = 0; r < 16; ++r) sb += acc[mb][nb][r];
                         const v2i sv = {(int)(uint32_t)(unsigned long long)sb, (int)(uint32_t)((unsigned long long)sb >> 32)};
-                        __builtin_amdgcn_raw_buffer_store_b64(sv, mine, ((mb * 16) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+                        __builtin_amdgcn_raw_buffer_store_b64(sv, mine, ((mb * 16) * NT + tid) * 16, 0, DEVICE_SCOPE);
                     }
                 }
             }
@@ -870,7 +877,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                     if (!(travelMb & (1u << mb))) {
                         if constexpr (RM) {
                             if (args.checksum != nullptr) {
-                                const v2i sv = __builtin_amdgcn_raw_buffer_load_b64(other, ((mb * 16) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+                                const v2i sv = __builtin_amdgcn_raw_buffer_load_b64(other, ((mb * 16) * NT + tid) * 16, 0, DEVICE_SCOPE);
                                 othersSum[mb] += (long long)(((unsigned long long)(uint32_t)sv.y << 32) | (uint32_t)sv.x);
                             }
                         }
@@ -881,7 +888,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
-                            pv[nb][g] = __builtin_amdgcn_raw_buffer_load_b128(other, (((mb * 4 + nb) * 4 + g) * 256 + tid) * 16, 0, DEVICE_SCOPE);
+                            pv[nb][g] = __builtin_amdgcn_raw_buffer_load_b128(other, (((mb * 4 + nb) * 4 + g) * NT + tid) * 16, 0, DEVICE_SCOPE);
 #pragma unroll
                     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
@@ -1008,7 +1015,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             if (tid < 2) {
                 long long t = 0;
 #pragma unroll
-                for (int i = 0; i < WM; ++i) t += red[2 * i + tid];
+                for (int i = 0; i < WR; ++i) t += red[2 * i + tid];
                 ((long long *)args.checksum)[(size_t)(ti.row / 128u) * (args.N / 128u) + ti.col / 128u + tid] = t;
             }
         }
@@ -1099,7 +1106,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             // buffers, five units (40 KiB per wave) in flight.  Every element sees the same additions in the same order as in
             // accumulator layout.
             static_assert(NW * 16384 <= POOL, "one 16 KiB staging area per wave");
-            constexpr int NBUF = 6;
+            constexpr int NBUF = W8 ? 4 : 6;   // (eight waves: 256 registers per wave; the count must be even)
             unsigned char *st = smem + w * 16384;
             __syncthreads();   // every wave has left the main loop's LDS reads behind
             const uint32_t U = 2u * nPeersF32;   // units: peer u / 2, rows 16 (u & 1) .. of the block
@@ -1349,7 +1356,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             Sum t = 0;
 #pragma unroll
             for (int i = 0; i < NW; ++i) t += red[i];
-            if constexpr (MB == 1) {
+            if constexpr (HALF) {
                 // The two 64-row halves of a task meet through a 64-bit word per task (the workspace's counter block, all zero
                 // between launches): each exchanges its sum, encoded so that it is never zero, into the word; the half that
                 // finds the other's sum there adds the two (either order gives the same bits), writes the task's checksum
@@ -1380,8 +1387,8 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
 }
 
 // One workgroup per tile, or per k slice of a tile.
-template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false, int NS = 3, bool PP = false, bool AQ = false>
-__global__ void __launch_bounds__(128 * WM, NS == 3 ? 2 : 1) gemm_dma_kernel(const GemmArgs args)
+template <uint32_t DT, int WM, bool TB = false, bool RM = false, bool RG = false, bool TA = false, int NS = 3, bool PP = false, bool AQ = false, bool W8 = false>
+__global__ void __launch_bounds__(128 * WM * (W8 ? 2 : 1), NS == 3 ? 2 : 1) gemm_dma_kernel(const GemmArgs args)
 {
     __shared__ __attribute__((aligned(1024))) unsigned char smem[DmaPool<WM, NS, AQ, TB>::BYTES];
     // A launch with few tiles can cut every tile's k range into kSlices pieces, one workgroup each (128-row tiles
@@ -1398,7 +1405,7 @@ __global__ void __launch_bounds__(128 * WM, NS == 3 ? 2 : 1) gemm_dma_kernel(con
             pos = blockIdx.x / kSlices;
         }
     }
-    dma_tile<DT, WM, TB, RM, RG, TA, 2, NS, PP, AQ>(args, smem, pos, slice, kSlices, 0);
+    dma_tile<DT, WM, TB, RM, RG, TA, W8 ? 1 : 2, NS, PP, AQ, W8>(args, smem, pos, slice, kSlices, 0);
 }
 
 // Reduce-scatter launches of a single round of workgroups (no more tiles than the 512 slots of the GPU) run some tiles as two

@@ -23,16 +23,23 @@ int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
     }
     if (args.flags & GF_ROW_MASK) {   // explicit kept rows in whole 32-row blocks
         const uint32_t wgs = launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u);
-        if (args.transB) {   // B as [n,k]: the three-stage and the six-stage ring
-            if (deep_ring(args, wgs, 1u))
-                hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, true, false, false, 6, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);
+        // Launches of at most one workgroup per CU whose operands stream from HBM run the six-stage ring (the whole LDS) on
+        // EIGHT waves, 32 rows of the tile each: two waves per SIMD overlap what a wave alone on its SIMD pays one after the
+        // other in every k step (barrier, LDS latency, copy issue).  Same box, variants alternating, K = N = 8192 with the
+        // library's own k slices, four -> eight waves: M = 256 41.5 -> 33.9 us, M = 512 60.6 -> 53.4, M = 1024 98.4 -> 92.4
+        // (B as [n,k]: 43.7 -> 36.4, 66.4 -> 59.3, 112.2 -> 104.9).  A goes in pairs of k steps from 128 steps per workgroup
+        // on (K = 16384, M = 512, one / two slices: 142.5 -> 121.1 / 85.5 -> 83.2 us; shorter loops lose 2-5 % with pairs).
+        if (deep_ring(args, wgs, 1u)) {
+            const uint32_t stepsPerWg = args.K / 64u / (args.splitK > 1 ? args.splitK : 1u);
+            if (args.transB)
+                hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, true, false, false, 6, true, false, true>), dim3(wgs), dim3(512), 0, (hipStream_t)stream, args);
+            else if (stepsPerWg >= 128u && deep_ring_pairs(args, 1u))
+                hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true, false, false, 6, true, true, true>), dim3(wgs), dim3(512), 0, (hipStream_t)stream, args);
             else
-                hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);
+                hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true, false, false, 6, true, false, true>), dim3(wgs), dim3(512), 0, (hipStream_t)stream, args);
         }
-        else if (deep_ring(args, wgs, 1u) && deep_ring_pairs(args, 1u))
-            hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true, false, false, 6, true, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);
-        else if (deep_ring(args, wgs, 1u))
-            hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true, false, false, 6, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);
+        else if (args.transB)
+            hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);
         else
             hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true>), dim3(wgs), dim3(256), 0, (hipStream_t)stream, args);
         return (int)hipGetLastError();

@@ -1762,14 +1762,17 @@ def test_quant_config5_full_size(M):
     assert np.array_equal(host16(out), want), "kept rows differ from the oracle"
 
 
-@pytest.mark.parametrize("case", [(1024, 16, 0, 64, 8192), (512, 8, 448, 64, 8192), (768, 3, 256, 96, 8192),
-                                  (128, 4, 64, 32, 8192),      # eight k slices of 16 steps: the shortest range that runs A in pairs
+@pytest.mark.parametrize("case", [(1024, 16, 0, 64, 8192),     # whole tiles, 128 k steps per workgroup: A copied in pairs of steps
+                                  (512, 8, 448, 64, 8192), (768, 3, 256, 96, 8192),
+                                  (128, 4, 64, 32, 8192),      # eight k slices of 16 steps
+                                  (512, 8, 64, 64, 16384),     # two k slices of 128 steps: A in pairs with k slices
                                   (1024, 8, 128, 128, 8256)])  # an odd number of k steps: A step by step
 def test_quant_explicit_kept_rows_large_tiles_streamed_operands(case):
-    """Explicit kept rows on the 128x256 tiles with operands that stream from HBM (K = N = 8192): six-stage ring, the peers'
-    partials in row layout through the ring of register buffers, A copied in pairs of k steps where the k range allows --
-    with 15, 7, 3 and 2 peers, kept rows at the start, at the end and in the middle of A, whole tiles and k slices.  Kept rows bit for bit against the oracle, the other rows through the
-    per-block checksums."""
+    """Explicit kept rows on the 128x256 tiles with operands that stream from HBM (K = 8192 or more, N = 8192): six-stage ring
+    on eight waves, the peers' partials in row layout through the ring of register buffers, A copied in pairs of k steps
+    where a workgroup's k range is long enough -- with 15, 7, 3 and 2 peers, kept rows at the start, at the end and in the
+    middle of A, whole tiles and k slices.  Kept rows bit for bit against the oracle, the other rows through the per-block
+    checksums."""
     _need_gpu()
     M, P, kb, kr, K = case
     N = 8192
