@@ -815,6 +815,26 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
                 if ((ti.row + wm * 32 * MB + mb * 32 - args.keptBegin) < args.keptRows) travelMb |= 1u << mb;
         }
     }
+    // RM with the pipelined peer loads (launches of one round of workgroups): the kept tiles are few, and what ends the launch
+    // is the one workgroup per kept tile that streams the peers' partials of its kept rows through one CU (about 60 GB/s).
+    // Every other workgroup of the same tile column -- the tiles of the other row blocks and the k slices that do not
+    // finish the kept tile -- is done at about the moment that stream starts.  On its way out it reads one word of every
+    // 128-byte line of ONE peer's kept rows in its 256 columns (workgroup number u of the column takes peer nPeers - 1 - u:
+    // the stream starts at peer 0), so that the line is in the L2 (same XCD) or at least in the memory-side cache when the
+    // stream arrives there.  Nothing is done with the words.
+    auto prefetch_peers = [&]() {
+        if constexpr (RM && PP) {
+            const uint32_t lines = args.keptRows * 8u;   // of one peer's kept rows in this tile's columns
+            const uint32_t u = (ti.row / (uint32_t)BM) * kSlices + slice;
+            if (args.nPeers == 0 || (args.flags & GF_REDUCE_INT32) || u >= args.nPeers || lines > 8u * NT) return;
+            const float *peer = (const float *)args.peers[args.nPeers - 1u - u] + args.peerRowOffset * args.peerLd + ti.col;
+            for (uint32_t l = tid; l < lines; l += NT) {
+                const float word = *(volatile const float *)(peer + (size_t)(l >> 3) * args.peerLd + (l & 7u) * 32u);
+                (void)word;
+            }
+            CATCOC_WAIT_VMCNT(0);
+        }
+    };
     if constexpr (WM == 2) {
         if (kSlices > 1) {
             constexpr int DEVICE_SCOPE = 16;   // sc1
@@ -849,7 +869,10 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
             volatile uint32_t *flag = (volatile uint32_t *)smem;
             if (tid == 0) *flag = __hip_atomic_fetch_add(args.skCount + task, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
-            if (*flag != kSlices - 1u) return;
+            if (*flag != kSlices - 1u) {
+                prefetch_peers();
+                return;
+            }
             if (tid == 0) __hip_atomic_store(args.skCount + task, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             // Integer partials add exactly in any order, and so do two float partials: the last slice to arrive keeps its own in
             // registers and adds the others.  Three or more float partials are added in SLICE order whichever slice arrives
@@ -926,6 +949,7 @@ __device__ __forceinline__ void dma_tile(const GemmArgs &args, unsigned char *sm
         for (int mb = 0; mb < MB; ++mb)
             if ((ti.row + wm * 32 * MB + mb * 32 - args.keptBegin) < args.keptRows) keptMb |= 1u << mb;
         kept = ti.row < args.keptBegin + args.keptRows && ti.row + BM > args.keptBegin;
+        if (!kept) prefetch_peers();
     }
     // W8A8 accumulators are dequantised in place (the registers then hold fp32 bit patterns); element accesses go
     // through scalar temporaries
