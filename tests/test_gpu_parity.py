@@ -1811,6 +1811,56 @@ def test_quant_explicit_kept_rows_large_tiles_streamed_operands(case):
             ops.quant_matmul_splitk(x1, x2, s1, s2, None, peers, P, kb, kr, workspace=None, n0=256, split_k=f)
 
 
+@pytest.mark.parametrize("case", [(256, 256, 64, 2, 0, 32, 1, False, False, True), (256, 512, 128, 8, 32, 32, 2, True, False, True),
+                                  (384, 512, 192, 4, 96, 96, 3, False, True, False), (256, 512, 448, 16, 224, 32, 2, True, True, True),
+                                  (512, 256, 1088, 8, 448, 64, 4, False, False, False), (256, 768, 320, 3, 64, 128, 1, True, False, False),
+                                  (1024, 512, 832, 8, 128, 128, 0, False, False, False)])
+def test_quant_explicit_kept_rows_eight_wave_ring_short_k_ranges(case):
+    """Explicit kept rows on the 128x256 tiles at sizes where a workgroup's k range is shorter than the six-stage ring, odd, or
+    unequal between the k slices (1 to 17 steps of 64): eight waves per workgroup, both layouts of B, fp32 and int32 peers at a
+    row offset, with and without a dump of the accumulators (without one only the kept 32-row blocks travel between the
+    slices).  Everything the launch writes against the oracle: accumulators, kept int32 block, output, checksums per
+    128 x 128 block of the rows that are not kept."""
+    _need_gpu()
+    M, N, K, P, kb, kr, f, tb, ri, dump = case
+    rng = np.random.default_rng(770 + M + K)
+    x1 = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    x2 = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    s1 = rng.uniform(0.005, 0.02, M).astype(np.float32)
+    s2 = rng.uniform(0.001, 0.01, N).astype(np.float32)
+    b = rng.integers(-1000, 1000, N, dtype=np.int32)
+    pro = 5
+    peers = [rng.integers(-2 ** 24, 2 ** 24, (kr, N), dtype=np.int32) if ri else rng.standard_normal((kr, N)).astype(np.float32) for _ in range(P - 1)]
+    staged = [np.concatenate([np.full((pro, N), 77, p.dtype), p]) for p in peers]
+    acc_want, out_want = oracle.quant_matmul_reduce_scatter(x1, x2, s1, s2, b, kb, kr, peers, oracle.BF16, reduce_int32=ri)
+    need, fac, blocks = ops.splitk_plan(M, K, N, P, kb, kr, n0=256, split_k=f)
+    assert blocks == (M // 128) * (N // 128) and (f == 0 or fac == f)
+    ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=DEV)
+    acc_dump = torch.full((M, N), -7, dtype=torch.int32, device=DEV) if dump else None
+    c_accum = torch.full((kr, N), -7, dtype=torch.int32, device=DEV)
+    checksum = torch.zeros(blocks, dtype=torch.int64, device=DEV)
+    x2d = dev(np.ascontiguousarray(x2.T)) if tb else dev(x2)
+    launch, out = ops.prepare_quant_matmul_splitk(dev(x1), x2d, dev(s1), dev(s2), dev(b), [dev(p) for p in staged], P, kb, kr, checksum=checksum,
+                                                  acc_dump=acc_dump, c_accum=c_accum, trans_b=tb, reduce_int32=ri, n0=256, split_k=f,
+                                                  workspace=ws, peer_row_offset=pro)
+    keep = np.zeros(M, bool)
+    keep[kb:kb + kr] = True
+    want_cs = np.array([[acc_want[mi * 128:(mi + 1) * 128, ni * 128:(ni + 1) * 128].astype(np.int64)[~keep[mi * 128:(mi + 1) * 128]].sum()
+                         for ni in range(N // 128)] for mi in range(M // 128)])
+    for it in range(2):   # (twice: the counters of the k slices go back to zero)
+        out.zero_()
+        checksum.zero_()
+        launch()
+        L.check()
+        torch.cuda.synchronize()
+        if dump:
+            assert np.array_equal(acc_dump.cpu().numpy(), acc_want), "int32 accumulators differ from the oracle"
+        assert np.array_equal(c_accum.cpu().numpy(), acc_want[kb:kb + kr] + (sum(peers) if ri else 0)), "kept int32 block differs"
+        assert np.array_equal(host16(out), out_want), "kept rows differ from the oracle"
+        assert np.array_equal(checksum.cpu().numpy().reshape(M // 128, N // 128), want_cs)
+    assert not ws[:65536].any()
+
+
 # ------------------------------------------------------- C ABI from a plain C++ host
 def test_launches_replay_from_a_hip_graph():
     # serving loops capture their launches: the library allocates nothing and never synchronises, the split-K path
