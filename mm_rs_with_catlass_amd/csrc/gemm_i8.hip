@@ -23,8 +23,8 @@ int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
     }
     if (args.flags & GF_ROW_MASK) {   // explicit kept rows in whole 32-row blocks
         const uint32_t wgs = launch_positions(args) * (args.splitK > 1 ? args.splitK : 1u);
-        // Launches of at most one workgroup per CU run the six-stage ring (the whole LDS of the CU) on EIGHT waves, 32 rows
-        // of the tile each, with the peers' partials pipelined through register buffers:
+        // Launches of at most 512 workgroups (one or two rounds of one workgroup per CU) run the six-stage ring (the whole
+        // LDS of the CU) on EIGHT waves, 32 rows of the tile each, with the peers' partials pipelined through register buffers:
         //  - two waves per SIMD overlap what a wave alone on its SIMD pays one after the other in every k step (barrier, LDS
         //    latency, copy issue).  Same box, variants alternating, K = N = 8192, operands from HBM, the library's own k
         //    slices, four -> eight waves: M = 256 41.5 -> 33.9 us, M = 512 60.6 -> 53.4, M = 1024 98.4 -> 92.4 (B as [n,k]:
@@ -33,9 +33,11 @@ int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
         //    registers (the three-stage kernel) it takes 35 us at M = 512 with seven peers, pipelined 8-10.  Three-stage
         //    kernel -> this one, operands of less than 48 MB: M = 512, K = 4096 / 2048 79.9 -> 35.9 / 70.8 -> 27.4 us,
         //    M = 256, K = 4096 74.7 -> 24.8, M = 1024, K = 2048 80.2 -> 42.0, M = 512, K = 8192, N = 4096 81.7 -> 36.9.
+        // More workgroups, eight-wave ring against the three-stage kernel with two workgroups per CU (K = N = 8192): 384 (M = 1536)
+        // 156.1 -> 142.1 us, 512 (M = 512 in four k slices / M = 2048) 102.6 -> 55.8 / 174.7 -> 168.0, 1024 (M = 4096) 293.3 -> 334.2.
         // A goes in pairs of k steps from 128 steps per workgroup on (K = 16384, M = 512, one / two slices: 142.5 -> 121.1 /
         // 85.5 -> 83.2 us; shorter loops lose 2-5 % with pairs).
-        if (wgs <= 256u) {
+        if (wgs <= 512u) {
             const uint32_t stepsPerWg = args.K / 64u / (args.splitK > 1 ? args.splitK : 1u);
             if (args.transB)
                 hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, true, false, false, 6, true, false, true>), dim3(wgs), dim3(512), 0, (hipStream_t)stream, args);
