@@ -36,12 +36,15 @@ int launch_gemm_dma_i8(const GemmArgs &args, void *stream)
         // More workgroups, eight-wave ring against the three-stage kernel with two workgroups per CU (K = N = 8192): 384 (M = 1536)
         // 156.1 -> 142.1 us, 512 (M = 512 in four k slices / M = 2048) 102.6 -> 55.8 / 174.7 -> 168.0, 1024 (M = 4096) 293.3 -> 334.2.
         // A goes in pairs of k steps from 128 steps per workgroup on (K = 16384, M = 512, one / two slices: 142.5 -> 121.1 /
-        // 85.5 -> 83.2 us; shorter loops lose 2-5 % with pairs).
+        // 85.5 -> 83.2 us; B as [n,k] 152.6 -> 139.0 / 106.4 -> 96.6; shorter loops lose 2-5 % with pairs).
         if (wgs <= 512u) {
             const uint32_t stepsPerWg = args.K / 64u / (args.splitK > 1 ? args.splitK : 1u);
-            if (args.transB)
+            const bool pairs = stepsPerWg >= 128u && deep_ring_pairs(args, 1u);
+            if (args.transB && pairs)
+                hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, true, false, false, 6, true, true, true>), dim3(wgs), dim3(512), 0, (hipStream_t)stream, args);
+            else if (args.transB)
                 hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, true, true, false, false, 6, true, false, true>), dim3(wgs), dim3(512), 0, (hipStream_t)stream, args);
-            else if (stepsPerWg >= 128u && deep_ring_pairs(args, 1u))
+            else if (pairs)
                 hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true, false, false, 6, true, true, true>), dim3(wgs), dim3(512), 0, (hipStream_t)stream, args);
             else
                 hipLaunchKernelGGL((gemm_dma_kernel<DT_I8, 2, false, true, false, false, 6, true, false, true>), dim3(wgs), dim3(512), 0, (hipStream_t)stream, args);

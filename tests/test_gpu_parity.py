@@ -1814,10 +1814,13 @@ def test_quant_explicit_kept_rows_large_tiles_streamed_operands(case):
 @pytest.mark.parametrize("case", [(256, 256, 64, 2, 0, 32, 1, False, False, True), (256, 512, 128, 8, 32, 32, 2, True, False, True),
                                   (384, 512, 192, 4, 96, 96, 3, False, True, False), (256, 512, 448, 16, 224, 32, 2, True, True, True),
                                   (512, 256, 1088, 8, 448, 64, 4, False, False, False), (256, 768, 320, 3, 64, 128, 1, True, False, False),
-                                  (1024, 512, 832, 8, 128, 128, 0, False, False, False)])
+                                  (1024, 512, 832, 8, 128, 128, 0, False, False, False),
+                                  (256, 256, 8192, 8, 32, 32, 1, True, False, False),      # 128 steps: A in pairs, B as [n,k]
+                                  (256, 512, 16384, 4, 64, 64, 2, False, True, True)])     # two slices of 128 steps: A in pairs
 def test_quant_explicit_kept_rows_eight_wave_ring_short_k_ranges(case):
     """Explicit kept rows on the 128x256 tiles at sizes where a workgroup's k range is shorter than the six-stage ring, odd, or
-    unequal between the k slices (1 to 17 steps of 64): eight waves per workgroup, both layouts of B, fp32 and int32 peers at a
+    unequal between the k slices (1 to 17 steps of 64), and two where it is long enough for A to be copied in pairs of steps:
+    eight waves per workgroup, both layouts of B, fp32 and int32 peers at a
     row offset, with and without a dump of the accumulators (without one only the kept 32-row blocks travel between the
     slices).  Everything the launch writes against the oracle: accumulators, kept int32 block, output, checksums per
     128 x 128 block of the rows that are not kept."""
