@@ -1897,6 +1897,14 @@ def test_launches_replay_from_a_hip_graph():
     csh = torch.zeros(512, dtype=torch.int64, device=DEV)
     wsh = torch.zeros(65536, dtype=torch.uint8, device=DEV)
     halves, out_halves = ops.prepare_quant_matmul_reduce_scatter(xh, wh, sh1, sh2, None, ph, 3, 8, checksum=csh, workspace=wsh)
+    # explicit kept rows on the 128x256 tiles in two k slices: the eight-wave ring, whose slices meet through tile counters
+    xr = torch.randint(-127, 128, (256, 2048), dtype=torch.int8, device=DEV, generator=g)
+    sr1 = torch.empty(256, device=DEV).uniform_(0.005, 0.02, generator=g)
+    pr = [torch.randn((32, N), device=DEV, generator=g) for _ in range(P - 1)]
+    need_r, fac_r, _ = ops.splitk_plan(256, 2048, N, P, 32, 32, n0=256, split_k=2)
+    assert fac_r == 2
+    wsr = torch.zeros(need_r, dtype=torch.uint8, device=DEV)
+    ring, out_ring = ops.prepare_quant_matmul_splitk(xr, w, sr1, s2, None, pr, P, 32, 32, split_k=2, workspace=wsr, n0=256)
     # the round-pipelined W8A8 operator (three comm rounds on two streams) with its events in a plan of the caller's: the call
     # then creates nothing, and the second stream joins the capture through the plan's events
     ipeers = [torch.randint(-2 ** 20, 2 ** 20, (M // P, N), dtype=torch.int32, device=DEV, generator=g) for _ in range(P - 1)]
@@ -1912,9 +1920,13 @@ def test_launches_replay_from_a_hip_graph():
     def pipe():
         ops.pipelined_quant_matmul_reduce_scatter(x1, x2, s1, s2, None, ipeers, 1, P, obp, c_accum=cacc_pipe, tiling=tp, comm_stream=comm,
                                                   block_num=8, out=out_pipe, plan=plan)
-    big(); small(); strips(); halves(); pipe(); L.check()
+    big(); small(); strips(); halves(); ring(); pipe(); L.check()
     torch.cuda.synchronize()
     want_big, want_small, want_halves, want_cs = out_big.clone(), out_small.clone(), out_halves.clone(), csh.clone()
+    want_ring = out_ring.clone()
+    _, ring_oracle = oracle.quant_matmul_reduce_scatter(xr[32:64].cpu().numpy(), w.cpu().numpy(), sr1[32:64].cpu().numpy(), s2.cpu().numpy(),
+                                                        None, 0, 32, [p.cpu().numpy() for p in pr], oracle.BF16)
+    assert np.array_equal(host16(want_ring), ring_oracle)
     assert torch.equal(out_strips, want_small), "the two weight layouts give the same rows"
     want_pipe, want_cacc = out_pipe.clone(), cacc_pipe.clone()
     fused = ops.quant_matmul_reduce_scatter(x1, x2, s1, s2, None, ipeers, 1, P, reduce_int32=True)
@@ -1925,18 +1937,20 @@ def test_launches_replay_from_a_hip_graph():
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
-        big(); small(); strips(); halves(); pipe()     # warm the side stream before capture
+        big(); small(); strips(); halves(); ring(); pipe()     # warm the side stream before capture
         torch.cuda.synchronize()
         with torch.cuda.graph(graph, stream=side):
             out_big.zero_()
             out_small.zero_()
             out_strips.zero_()
             out_halves.zero_()
+            out_ring.zero_()
             csh.zero_()
             big()
             small()
             strips()
             halves()
+            ring()
             pipe()
     L.check()
     for _ in range(3):
@@ -1944,6 +1958,7 @@ def test_launches_replay_from_a_hip_graph():
         out_small.fill_(1.0)
         out_strips.fill_(1.0)
         out_halves.fill_(1.0)
+        out_ring.fill_(1.0)
         out_pipe.fill_(1.0)
         cacc_pipe.fill_(3)
         csh.fill_(7)
@@ -1952,6 +1967,7 @@ def test_launches_replay_from_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(out_big, want_big) and torch.equal(out_small, want_small) and torch.equal(out_strips, want_small)
         assert torch.equal(out_halves, want_halves) and torch.equal(csh, want_cs)
+        assert torch.equal(out_ring, want_ring) and not wsr[:65536].any()
         assert torch.equal(out_pipe, want_pipe) and torch.equal(cacc_pipe, want_cacc)
         assert not ws[:65536].any(), "tile counters were not re-armed"
         assert not wsh.any(), "the words the checksum halves meet through were not cleared"
